@@ -1,0 +1,238 @@
+/*
+ * sage_hip.h — C ABI of the MI355X (gfx950) compute backend for Sage's operator hot path.
+ *
+ * Every entry point replaces one device-side responsibility of the reference (ingim/sage); the
+ * reference interface it stands in for is cited as file:line under the reference's `src/`.
+ * The boundary is the operator `compute` call (ops.rs:79-101, dispatched from ops.rs:163-187):
+ * strided tensor descriptors in, a freshly written contiguous tensor out, status-code errors.
+ *
+ * Conventions
+ *  - Plain C: pointers, sizes, PODs.  No C++ or torch types cross this boundary.
+ *  - Every function returns an sg_status.  Nothing aborts; after a non-OK return
+ *    sg_last_error() describes it, and for SG_ERR_OOM sg_last_oom() gives {needed,total}
+ *    (error.rs:5-13, session/memory.rs:45-54).
+ *  - A context owns one device, one in-order HIP stream, the kernel cache and the allocator
+ *    (session/context.rs:25-52).  Launches are asynchronous on that stream; sg_memcpy_d2h and
+ *    sg_sync wait for it (session/device.rs:111-147 are blocking the same way).
+ *  - A context is not thread-safe (the reference threads `&mut Context` everywhere); distinct
+ *    contexts are independent.
+ *  - The library never frees or reallocates caller memory.  Outputs are allocated by the caller
+ *    with sg_alloc and passed in; op outputs must be dense row-major ("default strides",
+ *    shape.rs:45-54) at any element offset, as the reference's outputs are (tensor.rs:195-210).
+ *  - Strides and offsets count ELEMENTS, not bytes; stride 0 is a broadcast axis
+ *    (shape.rs:190-195, 239-279).  Index arithmetic is exact.
+ *  - Only 4-byte element types are computed on (SG_FLOAT, SG_INT, SG_UINT): the reference sizes
+ *    every buffer as numel*4 bytes (session/device.rs:75), so nothing else is safe there either.
+ *    Other dtypes yield SG_ERR_DTYPE.
+ */
+#ifndef SAGE_HIP_H
+#define SAGE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SG_MAX_RANK 8
+#define SG_MAX_MAP_INPUTS 16
+#define SG_MAX_EXPR 128
+/* Allocator capacity a default reference Context runs with: 1000 MiB (session/context.rs:49). */
+#define SG_REFERENCE_CAPACITY_BYTES (1000ull * 1024ull * 1024ull)
+
+typedef enum sg_status {
+    SG_OK = 0,
+    SG_ERR_OOM = 1,    /* Error::Memory(OutOfMemory{mem_needed,mem_total})  memory.rs:246-255 */
+    SG_ERR_DEVICE = 2, /* Error::Device(ocl::Error) -> a hipError_t / hiprtc failure          */
+    SG_ERR_SHAPE = 3,  /* Error::Shape / the reference's shape assert!/panic! sites            */
+    SG_ERR_DTYPE = 4,  /* the reference's dtype assert_eq! sites (map.rs:489, 869-870)         */
+    SG_ERR_ARG = 5     /* null pointer, bad enum, unsupported combination                      */
+} sg_status;
+
+/* Same order as the reference's DataType enum (tensor/data.rs:14-30). */
+typedef enum sg_dtype {
+    SG_CHAR = 0, SG_SHORT = 1, SG_INT = 2, SG_LONG = 3,
+    SG_UCHAR = 4, SG_USHORT = 5, SG_UINT = 6, SG_ULONG = 7,
+    SG_FLOAT = 8, SG_HALF = 9
+} sg_dtype;
+
+/* TensorDesc + Shape (tensor.rs:38-41, shape.rs:38-42) plus the device pointer of the buffer. */
+typedef struct sg_tensor {
+    void *base;                   /* device pointer of element 0 of the underlying buffer */
+    int32_t dtype;                /* sg_dtype */
+    int32_t rank;                 /* 1..SG_MAX_RANK */
+    int64_t extents[SG_MAX_RANK];
+    int64_t strides[SG_MAX_RANK]; /* elements; 0 = broadcast */
+    int64_t offset;               /* elements */
+} sg_tensor;
+
+typedef struct sg_ctx sg_ctx;
+
+/* ---- context, memory, transfers: session/context.rs:43-52, session/device.rs:45-191 ---------- */
+
+/* Context::with_device (context.rs:43-52) + Device::new (device.rs:45-70).  capacity_bytes bounds
+ * the bytes handed out by sg_alloc (Allocator::new capacity, memory.rs:173-180); 0 = no cap beyond
+ * the device.  The reference default is SG_REFERENCE_CAPACITY_BYTES. */
+int sg_ctx_create(int device_idx, uint64_t capacity_bytes, sg_ctx **out);
+int sg_ctx_destroy(sg_ctx *ctx);
+
+/* Context::alloc -> Pool::alloc -> Device::alloc_buffer (context.rs:119-137, memory.rs:353-362,
+ * device.rs:73-89).  Over-capacity -> SG_ERR_OOM with needed = (total+size)-capacity,
+ * total = bytes currently reserved (memory.rs:246-255).  Freed blocks are cached and reused on the
+ * context's single in-order stream; sg_trim returns the cache to the device. */
+int sg_alloc(sg_ctx *ctx, uint64_t nbytes, void **dptr);
+/* OpenClMemory::drop (memory.rs:685-692). */
+int sg_free(sg_ctx *ctx, void *dptr);
+int sg_trim(sg_ctx *ctx);
+/* Allocator::{mem_used,mem_total,mem_peak,capacity} (memory.rs:182-198), in bytes. */
+int sg_mem_stats(sg_ctx *ctx, uint64_t *used, uint64_t *reserved, uint64_t *peak, uint64_t *capacity);
+
+/* Buffer::write / Buffer::read (device.rs:111-147): blocking copies. */
+int sg_memcpy_h2d(sg_ctx *ctx, void *dst_dev, const void *src_host, uint64_t nbytes);
+int sg_memcpy_d2h(sg_ctx *ctx, void *dst_host, const void *src_dev, uint64_t nbytes);
+int sg_memcpy_d2d(sg_ctx *ctx, void *dst_dev, const void *src_dev, uint64_t nbytes);
+/* Buffer::fill (device.rs:149-164) as used by Tensor::fill_zero (tensor.rs:212): 32-bit pattern. */
+int sg_fill_u32(sg_ctx *ctx, void *dst_dev, uint32_t pattern, uint64_t count);
+/* Queue::finish.  sg_stream returns the context's hipStream_t so a caller can time with events. */
+int sg_sync(sg_ctx *ctx);
+void *sg_stream(sg_ctx *ctx);
+
+const char *sg_last_error(sg_ctx *ctx);
+int sg_last_oom(sg_ctx *ctx, uint64_t *needed, uint64_t *total);
+/* Number of distinct kernels built at run time so far (Context::kernels, context.rs:29-31). */
+int sg_kernel_cache_size(sg_ctx *ctx);
+
+/* ---- fused elementwise maps: ops/map.rs ------------------------------------------------------ */
+
+/* UnaryMap (map.rs:93-130), BinaryMap (map.rs:152-172), TernaryMap (map.rs:194-196): same order. */
+typedef enum sg_unary {
+    SG_U_COPY = 0, SG_U_ABS, SG_U_NEG, SG_U_RECIP, SG_U_LOG, SG_U_EXP, SG_U_SQRT, SG_U_SQUARE,
+    SG_U_ERF, SG_U_SIGN, SG_U_CEIL, SG_U_FLOOR, SG_U_ROUND,
+    SG_U_SIN, SG_U_SINH, SG_U_COS, SG_U_COSH, SG_U_TAN, SG_U_TANH,
+    SG_U_ASIN, SG_U_ASINH, SG_U_ACOS, SG_U_ACOSH, SG_U_ATAN, SG_U_ATANH,
+    SG_U_NOT, SG_U_CAST_INT, SG_U_CAST_FLOAT, SG_U__COUNT
+} sg_unary;
+typedef enum sg_binary {
+    SG_B_ADD = 0, SG_B_SUB, SG_B_DIV, SG_B_MUL, SG_B_MOD, SG_B_POW, SG_B_MIN, SG_B_MAX,
+    SG_B_AND, SG_B_OR, SG_B_EQ, SG_B_NE, SG_B_GT, SG_B_GE, SG_B_LT, SG_B_LE, SG_B__COUNT
+} sg_binary;
+typedef enum sg_ternary { SG_T_COND = 0, SG_T__COUNT } sg_ternary;
+
+typedef enum sg_expr_kind {
+    SG_EXPR_INPUT = 0,   /* StackElement::Input(idx)              map.rs:218-222 */
+    SG_EXPR_LITERAL = 1, /* NullaryMap::Literal  "(type)value"     map.rs:517-531 */
+    SG_EXPR_UNARY = 2,
+    SG_EXPR_BINARY = 3,
+    SG_EXPR_TERNARY = 4
+} sg_expr_kind;
+
+/* One element of VariadicMapOperator.expr (map.rs:199-222) in the same PREFIX order the reference
+ * stores it: an operator is followed by its operands, left to right (ops.rs:116-130). */
+typedef struct sg_expr {
+    int32_t kind;  /* sg_expr_kind */
+    int32_t op;    /* sg_unary / sg_binary / sg_ternary, or the input index for SG_EXPR_INPUT */
+    int32_t dtype; /* SG_EXPR_LITERAL: sg_dtype of the literal (SG_FLOAT, SG_INT or SG_UINT) */
+    uint32_t bits; /* SG_EXPR_LITERAL: the 32-bit pattern of the value */
+} sg_expr;
+
+/* {Nullary,Unary,Binary,Ternary,Variadic}MapOperator::compute via compile_map (map.rs:369-410,
+ * 898-921, 970-998, 1044-1078, 1101-1120, 1141-1175): out[gid] = expr(in_0[idx_0], ...), with idx_i
+ * from translate_id (core.rs:113-175).  All inputs must have out's extents (the reference
+ * broadcasts beforehand with Expand -> stride 0, map.rs:412-456).  Result dtype follows
+ * map.rs:464-470, 491-501 and is checked against out->dtype.  n_in may be 0 (nullary_map).
+ * SG_B_MOD returns SG_ERR_ARG: the reference emits `mod(a, b)`, which is not an OpenCL C function,
+ * so its kernel cannot be built either (map.rs:275; its test is disabled, map.rs:1603). */
+int sg_map(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_tensor *in, int n_in,
+           const sg_tensor *out);
+
+/* ---- reductions: ops/reduce.rs --------------------------------------------------------------- */
+
+typedef enum sg_reduce_op { SG_R_SUM = 0, SG_R_PROD = 1, SG_R_MAX = 2, SG_R_MIN = 3 } sg_reduce_op;
+typedef enum sg_reduce_arg_op { SG_RA_MAX = 0, SG_RA_MIN = 1 } sg_reduce_arg_op;
+/* The reference starts every accumulator at literal 0 (reduce.rs:282), so its max is
+ * max(0, true max), its min is min(0, true min) and its prod is 0.  SG_INIT_REF_ZERO reproduces
+ * that bit for bit; SG_INIT_IDENTITY uses -inf/+inf/1/0.  Sum is identical under both. */
+typedef enum sg_reduce_init { SG_INIT_REF_ZERO = 0, SG_INIT_IDENTITY = 1 } sg_reduce_init;
+
+/* ReduceOperator::compute (reduce.rs:258-325).  `out` extents must be reduced_extents(in, axes,
+ * preserve) for either value of preserve (reduce.rs:124-140): only numel and contiguity matter. */
+int sg_reduce(sg_ctx *ctx, int op, const int32_t *axes, int n_axes, int init_mode,
+              const sg_tensor *in, const sg_tensor *out);
+/* ReduceArgOperator::compute (reduce.rs:372-431): first extreme index wins ties; out is SG_UINT. */
+int sg_reduce_arg(sg_ctx *ctx, int op, int axis, const sg_tensor *in, const sg_tensor *out);
+
+/* ---- indexing kernels: ops/core.rs ----------------------------------------------------------- */
+
+/* Gather::compute (core.rs:655-718): out has ind's extents; ind is SG_UINT or SG_INT read as
+ * unsigned (core.rs:679) through its own strides (stride 0 allowed).  No bounds check on the
+ * reference; here an index >= x.extents[axis] is not detected either (caller's contract). */
+int sg_gather(sg_ctx *ctx, int axis, const sg_tensor *x, const sg_tensor *ind, const sg_tensor *out);
+/* Scatter::compute (core.rs:764-833): out is zero-filled, then out[.., ind, ..] += x.  The
+ * reference's update is a non-atomic read-modify-write, so duplicate indices race there; here the
+ * add is atomic (deterministic up to fp32 summation order).  ind must have default strides: the
+ * reference decomposes gid by ind's own strides (core.rs:770, 807-808). */
+int sg_scatter(sg_ctx *ctx, int axis, const sg_tensor *x, const sg_tensor *ind, const sg_tensor *out);
+/* Unslice::compute (core.rs:553-611): out zero-filled, x copied into [start, start+x.extents[axis]). */
+int sg_unslice(sg_ctx *ctx, int axis, int64_t start, const sg_tensor *x, const sg_tensor *out);
+/* Concat::compute (core.rs:892-934). */
+int sg_concat(sg_ctx *ctx, int axis, const sg_tensor *in, int n_in, const sg_tensor *out);
+
+/* ---- GEMM: ops/gemm.rs + ops/kernels/matmul_direct.opencl ------------------------------------ */
+
+typedef enum sg_act { SG_ACT_NONE = 0, SG_ACT_RELU = 1, SG_ACT_GELU_ERF = 2 } sg_act;
+
+/* Optional fused epilogue (no counterpart in the reference, which runs each of these as a separate
+ * full-size map launch after the GEMM: layers.rs:243-247, nn.rs:33-40, bert.rs:203,279):
+ *   v = alpha * (A.B)[m,n];  v += bias[n];  v = act(v);  v += residual[m,n];  v = act_post(v).
+ * A null sg_gemm_epilogue* means alpha = 1 and nothing else, i.e. exactly the reference's GEMM
+ * (alpha = 1, beta = 0, gemm.rs:227-228). */
+typedef struct sg_gemm_epilogue {
+    float alpha;
+    int32_t act;               /* sg_act, applied after bias */
+    int32_t act_post;          /* sg_act, applied after residual */
+    const sg_tensor *bias;     /* numel == N, unit stride, or NULL */
+    const sg_tensor *residual; /* same extents as C, last stride 1, or NULL */
+} sg_gemm_epilogue;
+
+/* Gemm::compute_direct (gemm.rs:176-250): a, b, c are rank 2; (m,k,n) are taken from the extents
+ * as gemm.rs:190-217 does for the four transpose modes; ld = strides[0] and the inner stride must
+ * be 1 (the reference organizes its inputs first, gemm.rs:111-112).  fp32 only. */
+int sg_gemm(sg_ctx *ctx, int transpose_a, int transpose_b, const sg_tensor *a, const sg_tensor *b,
+            const sg_tensor *c, const sg_gemm_epilogue *epi);
+/* GemmBatched::compute_direct (gemm.rs:338-421): rank 3, batch stride = strides[0], ld = strides[1]. */
+int sg_gemm_batched(sg_ctx *ctx, int transpose_a, int transpose_b, const sg_tensor *a,
+                    const sg_tensor *b, const sg_tensor *c, const sg_gemm_epilogue *epi);
+/* matmul_batched (gemm.rs:53-104) without its organize copies: a = [batch.., M, K],
+ * b = [batch.., K, N], c = [batch.., M, N] with up to two leading batch axes and arbitrary strides,
+ * provided each matrix has one unit stride among its two inner axes (c: the N axis).  This is how
+ * permuted attention heads (bert.rs:282-302) are consumed and produced in place. */
+int sg_matmul_strided(sg_ctx *ctx, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c,
+                      const sg_gemm_epilogue *epi);
+
+/* ---- convolution feeder: ops/conv.rs --------------------------------------------------------- */
+
+/* Im2col::compute (conv.rs:289-374): x [N,H,W,C] dense -> out [N,OH,OW,KH,KW,C], zero padding.
+ * Every pair is {w, h} as in the reference (conv.rs:83, 205-206). */
+int sg_im2col(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, const int32_t ker[2],
+              const int32_t stride[2], const int32_t pad[2], const int32_t dil[2]);
+
+/* ---- fused row operators: compositions of ops/nn.rs ------------------------------------------ */
+
+/* softmax over the last axis (nn.rs:42-56) of (x + addend): one pass instead of reduce(max),
+ * exp(x-m) map, reduce(sum), divide map.  x: last stride 1; addend: NULL or same extents with
+ * broadcast strides (the extended attention mask of bert.rs:304-314). */
+int sg_softmax_lastaxis(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *addend,
+                        const sg_tensor *out);
+/* softmax_cross_entropy (nn.rs:70-82): logits [B,C] f32, labels [B,1] uint/int, loss [B]. */
+int sg_softmax_cross_entropy(sg_ctx *ctx, const sg_tensor *logits, const sg_tensor *labels,
+                             const sg_tensor *loss);
+/* layer_norm over the last axis (nn.rs:84-100): (x-E[x]) / sqrt(E[x^2]-E[x]^2+eps) * gamma + beta.
+ * gamma, beta: numel 1 (the reference's LayerNorm holds [1] scalars, layers.rs:563-564) or numel C. */
+int sg_layer_norm_lastaxis(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *gamma,
+                           const sg_tensor *beta, float eps, const sg_tensor *out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SAGE_HIP_H */

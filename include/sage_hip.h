@@ -145,6 +145,14 @@ typedef struct sg_expr {
  * so its kernel cannot be built either (map.rs:275; its test is disabled, map.rs:1603). */
 int sg_map(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_tensor *in, int n_in,
            const sg_tensor *out);
+/* The kernel text sg_map would build for these operands (compile_map's return value,
+ * map.rs:369-410), without building or launching it; base pointers may be null.  Writes at most
+ * cap-1 bytes plus a terminator, and the dtype the expression yields.  ctx may be null. */
+int sg_map_source(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_tensor *in, int n_in,
+                  const sg_tensor *out, char *buf, uint64_t cap, int32_t *result_dtype);
+/* Compiles kernel text for gfx950 exactly as sg_map does (KernelProgram::new, device.rs:201-213)
+ * but loads nothing, so it needs no GPU.  On failure the build log goes to log_buf. */
+int sg_map_compile_only(const char *source, char *log_buf, uint64_t log_cap);
 
 /* ---- reductions: ops/reduce.rs --------------------------------------------------------------- */
 

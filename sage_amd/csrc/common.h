@@ -1,0 +1,103 @@
+// Shared host-side declarations of the gfx950 backend: context, error plumbing, tensor helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <map>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/sage_hip.h"
+
+struct sg_block {
+    uint64_t size;       // bytes held from the device for this block
+    uint64_t requested;  // bytes the caller asked for (what the capacity check counts)
+};
+
+struct sg_jit_kernel {
+    hipModule_t module;
+    hipFunction_t fn;
+};
+
+// Context (session/context.rs:25-36): device + stream + kernel cache + allocator.
+struct sg_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    int num_cus = 256;
+    // allocator: live blocks by pointer, cached free blocks by size
+    uint64_t capacity = 0;  // 0 = unbounded
+    uint64_t used = 0;      // bytes handed out
+    uint64_t reserved = 0;  // bytes held from the device (used + cached)
+    uint64_t peak = 0;
+    std::unordered_map<void *, sg_block> live;
+    std::multimap<uint64_t, void *> cache;
+    // run-time built kernels keyed by their full source text (session/context.rs:62-83)
+    std::unordered_map<std::string, sg_jit_kernel> jit;
+    // errors
+    std::string last_error;
+    uint64_t oom_needed = 0, oom_total = 0;
+};
+
+int sg_fail(sg_ctx *ctx, int code, const char *fmt, ...);
+
+#define SG_HIP(ctx, expr)                                                                          \
+    do {                                                                                           \
+        hipError_t e_ = (expr);                                                                    \
+        if (e_ != hipSuccess)                                                                      \
+            return sg_fail(ctx, SG_ERR_DEVICE, "%s failed: %s (%s:%d)", #expr,                    \
+                           hipGetErrorString(e_), __FILE__, __LINE__);                             \
+    } while (0)
+
+#define SG_CHECK_LAUNCH(ctx, what)                                                                 \
+    do {                                                                                           \
+        hipError_t e_ = hipGetLastError();                                                         \
+        if (e_ != hipSuccess)                                                                      \
+            return sg_fail(ctx, SG_ERR_DEVICE, "launch of %s failed: %s", what,                   \
+                           hipGetErrorString(e_));                                                 \
+    } while (0)
+
+static inline int64_t sg_numel(const sg_tensor *t) {
+    int64_t n = 1;
+    for (int i = 0; i < t->rank; ++i) n *= t->extents[i];
+    return n;
+}
+
+static inline bool sg_dtype_ok(int dt) { return dt == SG_FLOAT || dt == SG_INT || dt == SG_UINT; }
+
+// Shape::default_strides (shape.rs:45-54)
+static inline void sg_default_strides(const int64_t *ext, int rank, int64_t *out) {
+    int64_t size = 1;
+    for (int i = 0; i < rank; ++i) size *= ext[i];
+    for (int i = 0; i < rank; ++i) {
+        size /= ext[i] ? ext[i] : 1;
+        out[i] = size;
+    }
+}
+
+// Dense row-major at any offset.  Axes of extent 1 may carry any stride.
+static inline bool sg_is_dense(const sg_tensor *t) {
+    int64_t expect = 1;
+    for (int i = t->rank - 1; i >= 0; --i) {
+        if (t->extents[i] != 1 && t->strides[i] != expect) return false;
+        expect *= t->extents[i];
+    }
+    return true;
+}
+
+int sg_validate_tensor(sg_ctx *ctx, const sg_tensor *t, const char *name);
+
+// Magic-number unsigned division for n < 2^31: q = (umulhi(n, magic) + n) >> shift.
+struct sg_fastdiv {
+    uint32_t magic, shift;
+};
+static inline sg_fastdiv sg_make_fastdiv(uint32_t d) {
+    sg_fastdiv f;
+    uint32_t s = 0;
+    while (s < 32 && (1ull << s) < d) ++s;
+    f.shift = s;
+    f.magic = (uint32_t)(((1ull << 32) * ((1ull << s) - d)) / d + 1);
+    return f;
+}

@@ -1,0 +1,409 @@
+// fp32 GEMM on the CDNA4 matrix cores (v_mfma_f32_32x32x2_f32), LDS-tiled, for gfx950.
+//
+// Replaces the reference's GEMM path: Gemm::compute_direct / GemmBatched::compute_direct
+// (gemm.rs:176-250, 338-421) launching the vendored XgemmDirect kernels at 8x8 tiles with one
+// output per work-item (matmul_direct.opencl:514-709), plus the organize() copies the reference
+// needs in front of it (gemm.rs:111-112, 258-259) and the separate bias / activation / residual map
+// launches behind it (layers.rs:243-247).
+//
+// Design:
+//   * One workgroup = 4 wavefronts computes a BM x BN tile of C; a wavefront owns a
+//     (BM/WAVES_M) x (BN/WAVES_N) sub-tile as TM x TN accumulators of 32x32 (16 VGPRs each).
+//   * K is walked in slabs of 32.  A slab of A and of B is fetched from global memory with
+//     16-byte loads into registers while the previous slab is being multiplied, then written to
+//     LDS as As[k][m], Bs[k][n] — the layout in which one MFMA operand fetch is a conflict-free
+//     ds_read of 32 consecutive floats per half-wave.  Operands that are contiguous along k
+//     (row-major A, transposed B) are transposed on their way into LDS, so all four transpose
+//     modes, and arbitrarily strided batches, run the same inner loop without any pre-copy.
+//   * Workgroup ids are remapped so that the ids one XCD receives (id mod 8) cover a compact block
+//     of tiles, which keeps the A/B panels a tile group shares inside that XCD's L2.
+//   * The epilogue applies alpha, bias[n], activation and a residual while the accumulators are
+//     still in registers.
+// Accumulation order differs from the reference's sequential k (MFMA sums pairs of k, slabs in
+// order); the difference is fp32 rounding only and is covered by the 1e-3 GEMM tolerance.
+#include "common.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 32;
+constexpr int PAD = 4;
+constexpr int NTHREADS = 256;
+constexpr int NUM_XCD = 8;
+
+struct GemmP {
+    const float *A, *B;
+    float *C;
+    const float *bias, *res;
+    int M, N, K;
+    int64_t a_sm, a_sk, b_sk, b_sn, c_sm, r_sm;
+    int64_t a_sb0, a_sb1, b_sb0, b_sb1, c_sb0, c_sb1, r_sb0, r_sb1;
+    int nb1;  // batch index = b0 * nb1 + b1
+    int tiles_m, tiles_n;
+    float alpha;
+    int act, act_post;
+    int vec_a, vec_b;  // 16-byte loads are legal for this operand
+};
+
+__device__ __forceinline__ float apply_act(float v, int act) {
+    if (act == SG_ACT_RELU) return v > 0.0f ? v : 0.0f * v;  // (float)(v>0) * v, nn.rs:39
+    if (act == SG_ACT_GELU_ERF) return (v * 0.5f) * (erff(v / 1.41421356237309504880f) + 1.0f);
+    return v;
+}
+
+// Fetch a ROWS x BK slab (rows = m or n indices) into registers, then store it to LDS as [k][row].
+template <int ROWS, bool K_CONTIG> struct Slab {
+    static constexpr int NV = ROWS * BK / 4 / NTHREADS;  // float4 per thread
+    static constexpr int LD = ROWS + PAD;
+    float4 r[NV];
+
+    __device__ __forceinline__ void load(const float *base, int row0, int k0, int row_lim, int k_lim, int64_t s_row, int64_t s_k,
+                                         int vec_ok, int tid) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int f = tid + i * NTHREADS;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (K_CONTIG) {
+                const int kq = f % (BK / 4), row = f / (BK / 4);
+                const int gr = row0 + row, gk = k0 + kq * 4;
+                if (gr < row_lim) {
+                    const float *p = base + (int64_t)gr * s_row + gk;
+                    if (vec_ok && gk + 3 < k_lim) {
+                        v = *reinterpret_cast<const float4 *>(p);
+                    } else {
+                        if (gk + 0 < k_lim) v.x = p[0];
+                        if (gk + 1 < k_lim) v.y = p[1];
+                        if (gk + 2 < k_lim) v.z = p[2];
+                        if (gk + 3 < k_lim) v.w = p[3];
+                    }
+                }
+            } else {
+                const int rq = f % (ROWS / 4), k = f / (ROWS / 4);
+                const int gr = row0 + rq * 4, gk = k0 + k;
+                if (gk < k_lim) {
+                    const float *p = base + (int64_t)gk * s_k + gr;
+                    if (vec_ok && gr + 3 < row_lim) {
+                        v = *reinterpret_cast<const float4 *>(p);
+                    } else {
+                        if (gr + 0 < row_lim) v.x = p[0];
+                        if (gr + 1 < row_lim) v.y = p[1];
+                        if (gr + 2 < row_lim) v.z = p[2];
+                        if (gr + 3 < row_lim) v.w = p[3];
+                    }
+                }
+            }
+            r[i] = v;
+        }
+    }
+
+    __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int f = tid + i * NTHREADS;
+            if (K_CONTIG) {
+                const int kq = f % (BK / 4), row = f / (BK / 4);
+                lds[(kq * 4 + 0) * LD + row] = r[i].x;
+                lds[(kq * 4 + 1) * LD + row] = r[i].y;
+                lds[(kq * 4 + 2) * LD + row] = r[i].z;
+                lds[(kq * 4 + 3) * LD + row] = r[i].w;
+            } else {
+                const int rq = f % (ROWS / 4), k = f / (ROWS / 4);
+                *reinterpret_cast<float4 *>(&lds[k * LD + rq * 4]) = r[i];
+            }
+        }
+    }
+};
+
+template <int BM, int BN, int WAVES_M, bool A_KC, bool B_NC>
+__global__ void __launch_bounds__(NTHREADS) gemm_mfma_kernel(const GemmP p) {
+    constexpr int WAVES_N = 4 / WAVES_M;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int LDA = BM + PAD, LDB = BN + PAD;
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA block");
+    __shared__ __attribute__((aligned(16))) float As[BK * LDA];
+    __shared__ __attribute__((aligned(16))) float Bs[BK * LDB];
+
+    // ---- which tile: spread consecutive ids over XCDs, then walk tiles in groups of 8 tile-rows
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int pid = blockIdx.x;
+    {
+        const int per = (ntiles + NUM_XCD - 1) / NUM_XCD;
+        int tall = ntiles % NUM_XCD;
+        if (tall == 0) tall = NUM_XCD;
+        const int xcd = pid % NUM_XCD, local = pid / NUM_XCD;
+        pid = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+    }
+    constexpr int GROUP_M = 8;
+    const int in_group = GROUP_M * p.tiles_n;
+    const int group = pid / in_group;
+    const int first_m = group * GROUP_M;
+    const int gsize = min(p.tiles_m - first_m, GROUP_M);
+    const int tile_m = first_m + (pid % in_group) % gsize;
+    const int tile_n = (pid % in_group) / gsize;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int b0 = blockIdx.y / p.nb1, b1 = blockIdx.y % p.nb1;
+    const float *A = p.A + b0 * p.a_sb0 + b1 * p.a_sb1;
+    const float *B = p.B + b0 * p.b_sb0 + b1 * p.b_sb1;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    Slab<BM, A_KC> sa;
+    Slab<BN, !B_NC> sb;
+    sa.load(A, m0, 0, p.M, p.K, p.a_sm, p.a_sk, p.vec_a, tid);
+    sb.load(B, n0, 0, p.N, p.K, p.b_sn, p.b_sk, p.vec_b, tid);
+
+    const int a_col = wm * WM + (lane & 31), b_col = wn * WN + (lane & 31), khalf = lane >> 5;
+    for (int k0 = 0; k0 < p.K; k0 += BK) {
+        __syncthreads();
+        sa.store(As, tid);
+        sb.store(Bs, tid);
+        __syncthreads();
+        if (k0 + BK < p.K) {
+            sa.load(A, m0, k0 + BK, p.M, p.K, p.a_sm, p.a_sk, p.vec_a, tid);
+            sb.load(B, n0, k0 + BK, p.N, p.K, p.b_sn, p.b_sk, p.vec_b, tid);
+        }
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+            float a[TM], b[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) a[i] = As[(kk + khalf) * LDA + a_col + i * 32];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) b[j] = Bs[(kk + khalf) * LDB + b_col + j * 32];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+    }
+
+    // ---- epilogue: element r of a 32x32 block sits at row (r/4)*8 + (lane/32)*4 + r%4, col lane%32
+    float *C = p.C + b0 * p.c_sb0 + b1 * p.c_sb1;
+    const float *R = p.res ? p.res + b0 * p.r_sb0 + b1 * p.r_sb1 : nullptr;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int n = n0 + wn * WN + j * 32 + (lane & 31);
+        if (n >= p.N) continue;
+        const float bias = p.bias ? p.bias[n] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * WM + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
+                if (m < p.M) {
+                    float v = acc[i][j][r];
+                    if (p.alpha != 1.0f) v *= p.alpha;
+                    if (p.bias) v += bias;
+                    v = apply_act(v, p.act);
+                    if (R) v += R[(int64_t)m * p.r_sm + n];
+                    v = apply_act(v, p.act_post);
+                    C[(int64_t)m * p.c_sm + n] = v;
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WAVES_M>
+int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch), block(NTHREADS);
+    if (a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true>), grid, block, 0, ctx->stream, p);
+    else if (a_kc && !b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, false>), grid, block, 0, ctx->stream, p);
+    else if (!a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, true>), grid, block, 0, ctx->stream, p);
+    else hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, false>), grid, block, 0, ctx->stream, p);
+    SG_CHECK_LAUNCH(ctx, "gemm");
+    return SG_OK;
+}
+
+// Tile choice: the largest tile that still gives every CU at least one workgroup, preferring an
+// exact multiple of the CU count (no partially filled last round of workgroups).
+int launch_gemm(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
+    struct Cfg { int bm, bn; };
+    static const Cfg cfgs[] = {{128, 128}, {128, 96}, {128, 64}, {64, 64}};
+    const int64_t cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+    int best = 3;
+    double best_score = -1.0;
+    for (int c = 0; c < 4; ++c) {
+        const int64_t tm = (p.M + cfgs[c].bm - 1) / cfgs[c].bm, tn = (p.N + cfgs[c].bn - 1) / cfgs[c].bn;
+        const int64_t tiles = tm * tn * batch;
+        const int64_t rounds = (tiles + cus - 1) / cus;
+        // useful work / (rounds * cus * tile area): fill of the last round and of edge tiles
+        const double useful = (double)p.M * p.N * batch;
+        const double spent = (double)rounds * cus * cfgs[c].bm * cfgs[c].bn;
+        double score = useful / spent;
+        // larger tiles re-read less of A and B: small bonus
+        score *= 1.0 + 0.05 * (3 - c);
+        if (score > best_score) {
+            best_score = score;
+            best = c;
+        }
+    }
+    const char *force = getenv("SAGE_GEMM_TILE");
+    if (force && force[0] >= '0' && force[0] <= '3') best = force[0] - '0';
+    switch (best) {
+    case 0: return launch_cfg<128, 128, 2>(ctx, p, batch, a_kc, b_nc);
+    case 1: return launch_cfg<128, 96, 4>(ctx, p, batch, a_kc, b_nc);
+    case 2: return launch_cfg<128, 64, 2>(ctx, p, batch, a_kc, b_nc);
+    default: return launch_cfg<64, 64, 2>(ctx, p, batch, a_kc, b_nc);
+    }
+}
+
+bool ptr_aligned16(const float *p) { return ((uintptr_t)p) % 16 == 0; }
+
+// a: [b0,b1,M,K] strides (.., sm, sk) ; b: [b0,b1,K,N] ; c: [b0,b1,M,N]
+struct Mat {
+    const float *ptr;
+    int64_t sb0, sb1, s_row, s_col;
+};
+
+int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c, const sg_gemm_epilogue *epi) {
+    if (M < 1 || N < 1 || K < 1) return sg_fail(ctx, SG_ERR_SHAPE, "gemm: empty dimension");
+    // Which axis of each operand is the contiguous one.  An axis of extent 1 may carry any stride.
+    bool a_kc, b_nc;
+    if (a.s_col == 1) a_kc = true;
+    else if (a.s_row == 1) a_kc = false;
+    else if (K == 1) { a_kc = true; a.s_col = 1; }
+    else if (M == 1) { a_kc = false; a.s_row = 1; }
+    else return sg_fail(ctx, SG_ERR_SHAPE, "gemm: A needs a unit stride on one of its two axes");
+    if (b.s_col == 1) b_nc = true;
+    else if (b.s_row == 1) b_nc = false;
+    else if (N == 1) { b_nc = true; b.s_col = 1; }
+    else if (K == 1) { b_nc = false; b.s_row = 1; }
+    else return sg_fail(ctx, SG_ERR_SHAPE, "gemm: B needs a unit stride on one of its two axes");
+    if (c.s_col != 1 && N != 1) return sg_fail(ctx, SG_ERR_SHAPE, "gemm: C needs a unit stride on its last axis");
+    GemmP p{};
+    p.A = a.ptr; p.B = b.ptr; p.C = (float *)c.ptr;
+    p.M = M; p.N = N; p.K = K;
+    p.a_sm = a.s_row; p.a_sk = a.s_col; p.b_sk = b.s_row; p.b_sn = b.s_col; p.c_sm = c.s_row;
+    p.a_sb0 = a.sb0; p.a_sb1 = a.sb1; p.b_sb0 = b.sb0; p.b_sb1 = b.sb1; p.c_sb0 = c.sb0; p.c_sb1 = c.sb1;
+    p.nb1 = nb1;
+    p.alpha = 1.0f; p.act = SG_ACT_NONE; p.act_post = SG_ACT_NONE;
+    auto mult4 = [](int64_t v) { return v % 4 == 0; };
+    p.vec_a = ptr_aligned16(a.ptr) && mult4(a_kc ? p.a_sm : p.a_sk) && mult4(a.sb0) && mult4(a.sb1);
+    p.vec_b = ptr_aligned16(b.ptr) && mult4(b_nc ? p.b_sk : p.b_sn) && mult4(b.sb0) && mult4(b.sb1);
+    if (epi) {
+        p.alpha = epi->alpha;
+        p.act = epi->act; p.act_post = epi->act_post;
+        if (p.act < 0 || p.act > SG_ACT_GELU_ERF || p.act_post < 0 || p.act_post > SG_ACT_GELU_ERF) return sg_fail(ctx, SG_ERR_ARG, "gemm: unknown activation");
+        if (epi->bias) {
+            const sg_tensor *t = epi->bias;
+            int rc = sg_validate_tensor(ctx, t, "gemm bias");
+            if (rc != SG_OK) return rc;
+            if (t->dtype != SG_FLOAT) return sg_fail(ctx, SG_ERR_DTYPE, "gemm: bias must be fp32");
+            if (sg_numel(t) != N || !sg_is_dense(t)) return sg_fail(ctx, SG_ERR_SHAPE, "gemm: bias must be dense with N = %d elements", N);
+            p.bias = (const float *)t->base + t->offset;
+        }
+        if (epi->residual) {
+            const sg_tensor *t = epi->residual;
+            int rc = sg_validate_tensor(ctx, t, "gemm residual");
+            if (rc != SG_OK) return rc;
+            if (t->dtype != SG_FLOAT) return sg_fail(ctx, SG_ERR_DTYPE, "gemm: residual must be fp32");
+            // accepted layouts: [M,N] for a single matrix, or the same rank as C
+            const int r = t->rank;
+            if (r < 2 || t->extents[r - 1] != N || t->extents[r - 2] != M || (N != 1 && t->strides[r - 1] != 1))
+                return sg_fail(ctx, SG_ERR_SHAPE, "gemm: residual must be [..,M,N] with unit last stride");
+            int64_t lead = 1;
+            for (int i = 0; i < r - 2; ++i) lead *= t->extents[i];
+            if (lead != (int64_t)nb0 * nb1) return sg_fail(ctx, SG_ERR_SHAPE, "gemm: residual batch extents differ from C's");
+            p.res = (const float *)t->base + t->offset;
+            p.r_sm = t->strides[r - 2];
+            p.r_sb1 = r >= 3 ? t->strides[r - 3] : 0;
+            p.r_sb0 = r >= 4 ? t->strides[r - 4] : 0;
+            if (r == 3 && nb0 > 1) {  // a single batch axis on the residual while C has it in b0
+                p.r_sb0 = t->strides[0];
+                p.r_sb1 = 0;
+            }
+            if (r > 4) return sg_fail(ctx, SG_ERR_SHAPE, "gemm: residual rank above 4");
+        }
+    }
+    return launch_gemm(ctx, p, nb0 * nb1, a_kc, b_nc);
+}
+
+int check_f32(sg_ctx *ctx, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c, const char *who) {
+    int rc;
+    if ((rc = sg_validate_tensor(ctx, a, who)) != SG_OK) return rc;
+    if ((rc = sg_validate_tensor(ctx, b, who)) != SG_OK) return rc;
+    if ((rc = sg_validate_tensor(ctx, c, who)) != SG_OK) return rc;
+    if (a->dtype != SG_FLOAT || b->dtype != SG_FLOAT || c->dtype != SG_FLOAT) return sg_fail(ctx, SG_ERR_DTYPE, "%s: fp32 only", who);
+    return SG_OK;
+}
+
+}  // namespace
+
+extern "C" int sg_gemm(sg_ctx *ctx, int ta, int tb, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c,
+                       const sg_gemm_epilogue *epi) {
+    if (!ctx) return SG_ERR_ARG;
+    int rc = check_f32(ctx, a, b, c, "sg_gemm");
+    if (rc != SG_OK) return rc;
+    if (a->rank != 2 || b->rank != 2 || c->rank != 2) return sg_fail(ctx, SG_ERR_SHAPE, "sg_gemm: rank-2 tensors expected");
+    // (height, chan1, width, chan2) of gemm.rs:118-124
+    const int64_t M = a->extents[ta ? 1 : 0], K = a->extents[ta ? 0 : 1];
+    const int64_t N = b->extents[tb ? 0 : 1], K2 = b->extents[tb ? 1 : 0];
+    if (K != K2) return sg_fail(ctx, SG_ERR_SHAPE, "sg_gemm: inner dimensions %lld and %lld differ (gemm.rs:124)", (long long)K, (long long)K2);
+    if (c->extents[0] != M || c->extents[1] != N) return sg_fail(ctx, SG_ERR_SHAPE, "sg_gemm: C must be [%lld,%lld]", (long long)M, (long long)N);
+    // ld = strides[0]; the stored inner axis must be contiguous (gemm.rs:111-112 organizes first)
+    if ((a->extents[1] != 1 && a->strides[1] != 1) || (b->extents[1] != 1 && b->strides[1] != 1) || (c->extents[1] != 1 && c->strides[1] != 1))
+        return sg_fail(ctx, SG_ERR_SHAPE, "sg_gemm: operands must have a unit inner stride (use sg_matmul_strided for general layouts)");
+    Mat ma{(const float *)a->base + a->offset, 0, 0, ta ? 1 : a->strides[0], ta ? a->strides[0] : 1};
+    Mat mb{(const float *)b->base + b->offset, 0, 0, tb ? 1 : b->strides[0], tb ? b->strides[0] : 1};
+    Mat mc{(const float *)c->base + c->offset, 0, 0, c->strides[0], 1};
+    return run(ctx, (int)M, (int)N, (int)K, 1, 1, ma, mb, mc, epi);
+}
+
+extern "C" int sg_gemm_batched(sg_ctx *ctx, int ta, int tb, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c,
+                               const sg_gemm_epilogue *epi) {
+    if (!ctx) return SG_ERR_ARG;
+    int rc = check_f32(ctx, a, b, c, "sg_gemm_batched");
+    if (rc != SG_OK) return rc;
+    if (a->rank != 3 || b->rank != 3 || c->rank != 3) return sg_fail(ctx, SG_ERR_SHAPE, "sg_gemm_batched: rank-3 tensors expected");
+    const int64_t batch = a->extents[0];
+    const int64_t M = a->extents[ta ? 2 : 1], K = a->extents[ta ? 1 : 2];
+    const int64_t N = b->extents[tb ? 1 : 2], K2 = b->extents[tb ? 2 : 1];
+    if (b->extents[0] != batch || c->extents[0] != batch) return sg_fail(ctx, SG_ERR_SHAPE, "sg_gemm_batched: batch extents differ (gemm.rs:261)");
+    if (K != K2) return sg_fail(ctx, SG_ERR_SHAPE, "sg_gemm_batched: inner dimensions differ (gemm.rs:276)");
+    if (c->extents[1] != M || c->extents[2] != N) return sg_fail(ctx, SG_ERR_SHAPE, "sg_gemm_batched: C must be [%lld,%lld,%lld]", (long long)batch, (long long)M, (long long)N);
+    if ((a->extents[2] != 1 && a->strides[2] != 1) || (b->extents[2] != 1 && b->strides[2] != 1) || (c->extents[2] != 1 && c->strides[2] != 1))
+        return sg_fail(ctx, SG_ERR_SHAPE, "sg_gemm_batched: operands must have a unit inner stride");
+    Mat ma{(const float *)a->base + a->offset, a->strides[0], 0, ta ? 1 : a->strides[1], ta ? a->strides[1] : 1};
+    Mat mb{(const float *)b->base + b->offset, b->strides[0], 0, tb ? 1 : b->strides[1], tb ? b->strides[1] : 1};
+    Mat mc{(const float *)c->base + c->offset, c->strides[0], 0, c->strides[1], 1};
+    return run(ctx, (int)M, (int)N, (int)K, (int)batch, 1, ma, mb, mc, epi);
+}
+
+extern "C" int sg_matmul_strided(sg_ctx *ctx, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c, const sg_gemm_epilogue *epi) {
+    if (!ctx) return SG_ERR_ARG;
+    int rc = check_f32(ctx, a, b, c, "sg_matmul_strided");
+    if (rc != SG_OK) return rc;
+    const int r = a->rank;
+    if (r < 2 || r > 4 || b->rank != r || c->rank != r) return sg_fail(ctx, SG_ERR_SHAPE, "sg_matmul_strided: ranks must agree and be 2..4");
+    const int64_t M = a->extents[r - 2], K = a->extents[r - 1], N = b->extents[r - 1];
+    if (b->extents[r - 2] != K) return sg_fail(ctx, SG_ERR_SHAPE, "sg_matmul_strided: inner dimensions differ");
+    if (c->extents[r - 2] != M || c->extents[r - 1] != N) return sg_fail(ctx, SG_ERR_SHAPE, "sg_matmul_strided: C extents do not match");
+    int64_t nb[2] = {1, 1};
+    int64_t sa[2] = {0, 0}, sb[2] = {0, 0}, sc[2] = {0, 0};
+    for (int i = 0; i < r - 2; ++i) {
+        const int slot = 2 - (r - 2) + i;
+        if (b->extents[i] != a->extents[i] || c->extents[i] != a->extents[i]) return sg_fail(ctx, SG_ERR_SHAPE, "sg_matmul_strided: batch extents differ");
+        nb[slot] = a->extents[i];
+        sa[slot] = a->strides[i];
+        sb[slot] = b->strides[i];
+        sc[slot] = c->strides[i];
+    }
+    Mat ma{(const float *)a->base + a->offset, sa[0], sa[1], a->strides[r - 2], a->strides[r - 1]};
+    Mat mb{(const float *)b->base + b->offset, sb[0], sb[1], b->strides[r - 2], b->strides[r - 1]};
+    Mat mc{(const float *)c->base + c->offset, sc[0], sc[1], c->strides[r - 2], c->strides[r - 1]};
+    return run(ctx, (int)M, (int)N, (int)K, (int)nb[0], (int)nb[1], ma, mb, mc, epi);
+}

@@ -1,0 +1,189 @@
+"""Model-level parity: BERT (models/bert.rs) and ResNet-18 (models/resnet.rs) through the HIP path
+against the CPU oracle's op-for-op re-composition, and against an independent torch-CPU restatement.
+Tolerance rel 1e-3 (end-to-end model output)."""
+import numpy as np
+import pytest
+
+import sage_amd as S
+from oracle import oracle as O
+from sage_amd import var as V
+from sage_amd.bert import Bert, BertConfig, BertLayer
+from sage_amd.layers import load_params
+from sage_amd.resnet import ResNet, ResNetConfig
+from tests.util import REL_GEMM, close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = S.Context()
+    yield c
+    c.close()
+
+
+@pytest.fixture(autouse=True)
+def _fusion_on():
+    V.set_fusion(True)
+    yield
+    V.set_fusion(True)
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+
+
+def dev(ctx, a):
+    return S.Var.new(S.Tensor.from_numpy(ctx, a))
+
+
+def ht(a):
+    return O.HT.from_numpy(a)
+
+
+def bert_layer_params(rng, e, hdim, per_feature):
+    n = e if per_feature else 1
+    w = lambda i, o: (rng.standard_normal((i, o)) * 0.05).astype(np.float32)
+    v = lambda k: (rng.standard_normal((k,)) * 0.1).astype(np.float32)
+    ln = lambda: ((1.0 + 0.1 * rng.standard_normal((n,))).astype(np.float32), (0.1 * rng.standard_normal((n,))).astype(np.float32))
+    p = {"wk": w(e, e), "bk": v(e), "wq": w(e, e), "bq": v(e), "wv": w(e, e), "bv": v(e), "wo": w(e, e), "bo": v(e)}
+    p["ln1_g"], p["ln1_b"] = ln()
+    p["w1"], p["b1"], p["w2"], p["b2"] = w(e, hdim), v(hdim), w(hdim, e), v(e)
+    p["ln2_g"], p["ln2_b"] = ln()
+    return p
+
+
+def layer_param_list(p):
+    # BertLayer.params(): key, query, value, dense, norm ; ffn dense1, dense2 ; norm
+    return [p["wk"], p["bk"], p["wq"], p["bq"], p["wv"], p["bv"], p["wo"], p["bo"], p["ln1_g"], p["ln1_b"],
+            p["w1"], p["b1"], p["w2"], p["b2"], p["ln2_g"], p["ln2_b"]]
+
+
+def torch_bert_layer(x, mask, p, heads, act, eps):
+    import torch
+    t = lambda a: torch.from_numpy(np.asarray(a)).double()
+    x = t(x)
+    n, l, e = x.shape
+    d = e // heads
+    lin = lambda h, w, b: h @ t(w) + t(b)
+    sep = lambda h: h.view(n, l, heads, d).transpose(1, 2)
+    q, k, v = sep(lin(x, p["wq"], p["bq"])), sep(lin(x, p["wk"], p["bk"])), sep(lin(x, p["wv"], p["bv"]))
+    s = q @ k.transpose(-1, -2) / np.sqrt(d) + (1.0 - t(mask).view(n, 1, 1, l)) * -1e5
+    a = torch.softmax(s, -1) @ v
+    a = a.transpose(1, 2).reshape(n, l, e)
+
+    def lnorm(h, g, b):
+        m = h.mean(-1, keepdim=True)
+        var = (h * h).mean(-1, keepdim=True) - m * m
+        return (h - m) / torch.sqrt(var + eps) * t(g) + t(b)
+
+    h1 = lnorm(lin(a, p["wo"], p["bo"]) + x, p["ln1_g"], p["ln1_b"])
+    u = lin(h1, p["w1"], p["b1"])
+    u = torch.relu(u) if act == "relu" else 0.5 * u * (1 + torch.erf(u / np.sqrt(2.0)))
+    return lnorm(lin(u, p["w2"], p["b2"]) + h1, p["ln2_g"], p["ln2_b"]).numpy()
+
+
+@pytest.mark.parametrize("reference_exact", [True, False], ids=["reference_exact", "gelu_config"])
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "unfused"])
+def test_bert_layer(ctx, reference_exact, fused):
+    """BertLayer::pass (bert.rs:199-203) at n=2, l=24, e=64, 4 heads, ffn 160."""
+    say("bert layer", reference_exact, fused)
+    V.set_fusion(fused)
+    rng = np.random.default_rng(3)
+    n, l, e, heads, hdim = 2, 24, 64, 4, 160
+    cfg = BertConfig(e, 100, 64, hdim, 1, heads, 1e-12, 0.1, 2)
+    p = bert_layer_params(rng, e, hdim, per_feature=not reference_exact)
+    x = rng.standard_normal((n, l, e)).astype(np.float32)
+    mask = np.ones((n, l), np.float32)
+    mask[1, 17:] = 0.0
+    layer = BertLayer(cfg, reference_exact)
+    load_params(ctx, layer, layer_param_list(p))
+    n0 = ctx.launches
+    y = layer.pass_(dev(ctx, x), dev(ctx, mask)).eval(ctx).numpy()
+    launches = ctx.launches - n0
+    say("launches", launches)
+    act = "relu" if reference_exact else "gelu"
+    eps = 1e-5 if reference_exact else 1e-12
+    yo = O.bert_layer(ht(x), ht(mask), {k: ht(v) for k, v in p.items()}, heads, act, eps).numpy()
+    close(y, yo, REL_GEMM, "vs oracle")
+    close(y, torch_bert_layer(x, mask, p, heads, act, eps), REL_GEMM, "vs torch float64")
+    if fused:
+        assert launches <= 14, launches
+
+
+def test_bert_model_reference_exact(ctx):
+    """Bert::pass (bert.rs:72-81): embeddings -> 2 layers -> token 1 -> Dense."""
+    say("bert model")
+    rng = np.random.default_rng(5)
+    cfg = BertConfig(32, 50, 40, 64, 2, 2, 0.0, 0.0, 3)
+    n, l = 3, 12
+    model = Bert(cfg, reference_exact=True)
+    arrays = [(rng.standard_normal((50, 32))).astype(np.float32), rng.standard_normal((40, 32)).astype(np.float32),
+              np.ones(1, np.float32), np.ones(1, np.float32)]
+    layers = []
+    for _ in range(2):
+        p = bert_layer_params(rng, 32, 64, per_feature=False)
+        layers.append(p)
+        arrays += layer_param_list(p)
+    wc, bc = (rng.standard_normal((32, 3)) * 0.1).astype(np.float32), np.zeros(3, np.float32)
+    arrays += [wc, bc]
+    load_params(ctx, model, arrays)
+    ids = rng.integers(0, 50, (n, l)).astype(np.int32)
+    mask = np.ones((n, l), np.float32)
+    y = model.pass_(dev(ctx, ids), dev(ctx, mask), ctx).eval(ctx).numpy()
+    po = {"word_emb": ht(arrays[0]), "pos_emb": ht(arrays[1]), "emb_g": ht(arrays[2]), "emb_b": ht(arrays[3]),
+          "layers": [{k: ht(v) for k, v in p.items()} for p in layers], "wc": ht(wc), "bc": ht(bc)}
+    yo = O.bert_forward(ht(ids.view(np.uint32).astype(np.uint32)), ht(mask), po, 2).numpy()
+    assert y.shape == (n, 3)
+    close(y, yo, REL_GEMM, "bert vs oracle")
+
+
+def resnet_arrays(rng, chan_in, classes):
+    """Parameters in ResNet.params() order + the oracle's dict form.  Kaiming-normal filters
+    (std = sqrt(1/fan_in), tensor/init.rs:27-50), zero biases (layers.rs:373-381)."""
+    def conv(kh, kw, ci, co):
+        fan_in = kw * ci * co  # [d0=KH, d1=KW, rest=C*OC] -> fan_in = d1 * prod(rest)
+        return (rng.standard_normal((kh, kw, ci, co)) * np.sqrt(1.0 / fan_in) * 4).astype(np.float32)
+    arrays, blocks = [], []
+    w0 = conv(7, 7, chan_in, 64)
+    arrays += [w0, np.zeros(64, np.float32)]
+    inp, out = 64, 64
+    for i in range(4):
+        stride = 1 if i == 0 else 2
+        ip = inp
+        for b in range(2):
+            s = stride if b == 0 else 1
+            blk = {"stride": s, "w1": conv(3, 3, ip, out), "b1": (rng.standard_normal(out) * 0.05).astype(np.float32),
+                   "w2": conv(3, 3, out, out), "b2": (rng.standard_normal(out) * 0.05).astype(np.float32)}
+            arrays += [blk["w1"], blk["b1"], blk["w2"], blk["b2"]]
+            if s != 1 or ip != out:
+                blk["wd"], blk["bd"] = conv(1, 1, ip, out), np.zeros(out, np.float32)
+                arrays += [blk["wd"], blk["bd"]]
+            blocks.append(blk)
+            ip = out
+        inp = out
+        out *= 2
+    wfc = (rng.standard_normal((512, classes)) * 0.05).astype(np.float32)
+    bfc = np.zeros(classes, np.float32)
+    arrays += [wfc, bfc]
+    return arrays, {"w0": w0, "b0": arrays[1], "blocks": blocks, "wfc": wfc, "bfc": bfc}
+
+
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "unfused"])
+def test_resnet18(ctx, fused):
+    """ResNet::new(d18(1,10)) (resnet.rs:75-104) on [3,28,28,1]."""
+    say("resnet18", fused)
+    V.set_fusion(fused)
+    rng = np.random.default_rng(4)
+    arrays, po = resnet_arrays(rng, 1, 10)
+    model = ResNet(ResNetConfig.d18(1, 10))
+    load_params(ctx, model, arrays)
+    x = rng.uniform(0, 1, (3, 28, 28, 1)).astype(np.float32)
+    n0 = ctx.launches
+    y = model.pass_(dev(ctx, x)).eval(ctx).numpy()
+    say("launches", ctx.launches - n0)
+    conv = lambda d: {k: (ht(v) if isinstance(v, np.ndarray) else v) for k, v in d.items()}
+    pod = {"w0": ht(po["w0"]), "b0": ht(po["b0"]), "blocks": [conv(b) for b in po["blocks"]], "wfc": ht(po["wfc"]), "bfc": ht(po["bfc"])}
+    yo = O.resnet18_forward(ht(x), pod).numpy()
+    assert y.shape == (3, 10)
+    close(y, yo, REL_GEMM, "resnet vs oracle")

@@ -1,0 +1,540 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle on seeded random inputs.
+
+Bar: indexing, gather, argmax, compare/logic results and pure +,-,*,/ arithmetic are bit-exact;
+transcendental maps and reductions agree within rel 1e-4; GEMM, convolution and model outputs
+within rel 1e-3 (tests/util.py).  Every test prints its case before touching the GPU.
+"""
+import numpy as np
+import pytest
+
+import sage_amd as S
+from oracle import oracle as O
+from sage_amd import abi, nn
+from sage_amd import var as V
+from tests.util import REL_GEMM, REL_MAP, close, exact
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = S.Context()
+    yield c
+    c.close()
+
+
+@pytest.fixture(autouse=True)
+def _fusion_on():
+    V.set_fusion(True)
+    yield
+    V.set_fusion(True)
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+
+
+def dev(ctx, a):
+    return S.Var.new(S.Tensor.from_numpy(ctx, a))
+
+
+def ht(a):
+    return O.HT.from_numpy(a)
+
+
+def view_pair(ctx, a, fn):
+    """The same layout operation applied to a device Var and to an oracle host tensor."""
+    return fn(dev(ctx, a)), fn(ht(a))
+
+
+# ----------------------------------------------------------------------------- maps
+UNARY_DOMAIN = {
+    "log": (0.1, 4.0), "sqrt": (0.0, 4.0), "acosh": (1.0, 5.0), "atanh": (-0.95, 0.95),
+    "asin": (-1.0, 1.0), "acos": (-1.0, 1.0), "recip": (0.5, 3.0), "exp": (-5.0, 5.0),
+}
+EXACT_UNARY = {"copy", "abs", "neg", "recip", "sqrt", "square", "sign", "ceil", "floor", "round", "cast_int", "cast_float", "not"}
+
+
+@pytest.mark.parametrize("name", abi.UNARY)
+@pytest.mark.parametrize("shape", [(64, 256), (7, 13), (3, 5, 4)], ids=["vec", "odd", "rank3"])
+def test_unary_maps(ctx, name, shape):
+    say("unary", name, shape)
+    rng = np.random.default_rng(hash(name) % 1000)
+    lo, hi = UNARY_DOMAIN.get(name, (-3.0, 3.0))
+    x = rng.uniform(lo, hi, shape).astype(np.float32)
+    if name in ("sign", "ceil", "floor", "round", "abs"):
+        x.flat[:6] = [0.0, -0.0, 0.5, -0.5, 1.5, -2.5]
+    y = V.unary_map(dev(ctx, x), name).eval(ctx).numpy()
+    y_or = O.unary(name, ht(x)).numpy()
+    assert y.dtype == y_or.dtype
+    if name in EXACT_UNARY:
+        exact(y, y_or, name)
+    else:
+        close(y, y_or, REL_MAP, name)
+
+
+@pytest.mark.parametrize("name", [b for b in abi.BINARY if b != "mod"])
+def test_binary_maps_float(ctx, name):
+    say("binary float", name)
+    rng = np.random.default_rng(7)
+    a = rng.uniform(0.2, 3.0, (33, 20)).astype(np.float32)
+    b = rng.uniform(0.2, 3.0, (33, 20)).astype(np.float32)
+    b[::3] = a[::3]  # ties for the comparisons
+    y = V.binary_map(dev(ctx, a), dev(ctx, b), name).eval(ctx).numpy()
+    y_or = O.binary(name, ht(a), ht(b)).numpy()
+    assert y.dtype == y_or.dtype
+    if name == "pow":
+        close(y, y_or, REL_MAP, name)
+    else:
+        exact(y, y_or, name)
+
+
+@pytest.mark.parametrize("name", ["add", "sub", "mul", "div", "min", "max", "eq", "lt", "ge", "and", "or"])
+@pytest.mark.parametrize("dt", [np.int32, np.uint32])
+def test_binary_maps_int(ctx, name, dt):
+    say("binary int", name, dt.__name__)
+    rng = np.random.default_rng(11)
+    a = rng.integers(0 if dt == np.uint32 else -50, 50, (16, 12)).astype(dt)
+    b = rng.integers(1, 9, (16, 12)).astype(dt)
+    y = V.binary_map(dev(ctx, a), dev(ctx, b), name).eval(ctx).numpy()
+    exact(y, O.binary(name, ht(a), ht(b)).numpy(), name)
+
+
+def test_int_unary_and_casts(ctx):
+    say("int unary / casts")
+    a = np.array([[-7, 0, 3, 2147483647], [5, -1, 9, -2147483648]], dtype=np.int32)
+    for name in ("neg", "copy", "not", "cast_float", "cast_int"):
+        exact(V.unary_map(dev(ctx, a), name).eval(ctx).numpy(), O.unary(name, ht(a)).numpy(), name)
+    f = np.array([[-2.7, -0.2, 0.0, 0.9], [1.5, 2.5, 100.25, -100.75]], dtype=np.float32)
+    exact(V.unary_map(dev(ctx, f), "cast_int").eval(ctx).numpy(), np.trunc(f).astype(np.int32), "trunc toward zero")
+    u = np.array([[0, 1, 2, 4000000000]], dtype=np.uint32)
+    exact(V.unary_map(dev(ctx, u), "cast_float").eval(ctx).numpy(), O.unary("cast_float", ht(u)).numpy(), "uint->float")
+
+
+LAYOUTS = {
+    "transpose01": lambda t: t.transpose(0, 1),
+    "permute_201": lambda t: t.permute([2, 0, 1]),
+    "slice_mid": lambda t: t.slice(1, 1, 4),
+    "slice_last": lambda t: t.slice(2, 3, 11),
+    "row_broadcast": lambda t: t.slice(2, 0, 1).expand(list(t.extents)),
+    "col_broadcast": lambda t: t.slice(1, 0, 1).expand(list(t.extents)),
+    "index_expand": lambda t: t.index(0, 1).expand(list(t.extents)),
+}
+
+
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+def test_map_operand_layouts(ctx, layout):
+    """Every index-translation class: direct, permuted, offset windows, stride-0 broadcasts."""
+    say("layout", layout)
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal((6, 8, 12)).astype(np.float32)
+    xd, xo = view_pair(ctx, a, LAYOUTS[layout])
+    b = rng.standard_normal(tuple(xo.extents)).astype(np.float32)
+    exact(xd.copy().eval(ctx).numpy(), xo.numpy(), "copy")
+    yd = (xd * dev(ctx, b) + xd).eval(ctx).numpy()
+    yo = O.binary("add", O.binary("mul", xo, ht(b)), xo).numpy()
+    exact(yd, yo, "x*b+x")
+
+
+def test_map_vector_and_broadcast_paths(ctx):
+    """Shapes that take the 16-byte path: bias rows, per-row scalars, attention-mask broadcast."""
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((96, 128)).astype(np.float32)
+    bias = rng.standard_normal((128,)).astype(np.float32)
+    rowv = rng.standard_normal((96, 1)).astype(np.float32)
+    say("bias add")
+    exact((dev(ctx, x) + dev(ctx, bias)).eval(ctx).numpy(), x + bias, "x+bias")
+    say("exp(x - rowmax)")
+    y = (dev(ctx, x) - dev(ctx, rowv)).exp().eval(ctx).numpy()
+    close(y, O.unary("exp", O.binary("sub", ht(x), ht(rowv))).numpy(), REL_MAP, "exp(x-c)")
+    say("scores/8 + mask")
+    s = rng.standard_normal((4, 3, 16, 16)).astype(np.float32)
+    m = rng.integers(0, 2, (4, 16)).astype(np.float32)
+    md = (-dev(ctx, m).view([4, 1, 1, 16]) + 1.0) * -1e5
+    mo = O.binary("mul", O.binary("add", O.unary("neg", ht(m).view([4, 1, 1, 16])), 1.0), -1e5)
+    exact((dev(ctx, s) / 8.0 + md).eval(ctx).numpy(), O.binary("add", O.binary("div", ht(s), 8.0), mo).numpy(), "s/8+mask")
+    say("five-input layer-norm tail")
+    mean = rng.standard_normal((96, 1)).astype(np.float32)
+    den = rng.uniform(0.5, 2.0, (96, 1)).astype(np.float32)
+    g, b = np.float32(1.5), np.float32(-0.25)
+    yd = ((dev(ctx, x) - dev(ctx, mean)) / dev(ctx, den) * dev(ctx, np.array([g])) + dev(ctx, np.array([b]))).eval(ctx).numpy()
+    exact(yd, ((x - mean) / den * g + b).astype(np.float32), "ln tail")
+
+
+def test_map_errors(ctx):
+    say("map error behaviour")
+    a = dev(ctx, np.ones((2, 3), np.float32))
+    i = dev(ctx, np.ones((2, 3), np.int32))
+    with pytest.raises(abi.DTypeError):
+        V.binary_map(a, i, "add")          # map.rs:489
+    with pytest.raises(abi.DTypeError):
+        V.cond(a, a, a)                    # map.rs:870: condition must be uint
+    with pytest.raises(abi.SageError):
+        V.binary_map(a, a, "mod").eval(ctx)  # map.rs:275: mod() cannot be built
+    with pytest.raises(ValueError):
+        V.binary_map(a, dev(ctx, np.ones((2, 4), np.float32)), "add")  # shape::union InvalidBroadcast
+
+
+def test_fused_map_equals_unfused(ctx):
+    say("fused vs unfused map chain")
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((40, 64)).astype(np.float32)
+    y = rng.uniform(0.5, 2.0, (40, 64)).astype(np.float32)
+
+    def build():
+        a, b = dev(ctx, x), dev(ctx, y)
+        return V.cond(V.gt(a, 0.0), (a * b + 1.0).sqrt() / b, -a.abs() * 0.5)
+
+    n0 = ctx.launches
+    f = build().eval(ctx).numpy()
+    assert ctx.launches - n0 == 1
+    V.set_fusion(False)
+    u = build().eval(ctx).numpy()
+    exact(f, u, "fusion changes no value")
+
+
+# ----------------------------------------------------------------------------- reductions
+RED_CASES = [
+    ((8, 1024), [1]), ((8, 1024), [0]), ((5, 37), [1]), ((3, 5000), [1]), ((64, 9, 32), [1]),
+    ((2, 3, 2, 3, 2), [0, 2, 3]), ((6, 7, 8), [0, 1, 2]), ((4, 6, 10), [2, 0]), ((128, 128), [1]), ((1, 7), [0]),
+]
+
+
+@pytest.mark.parametrize("op", ["sum", "prod", "max", "min"])
+@pytest.mark.parametrize("init", ["ref_zero", "identity"])
+@pytest.mark.parametrize("case", range(len(RED_CASES)))
+def test_reduce(ctx, op, init, case):
+    shape, axes = RED_CASES[case]
+    say("reduce", op, init, shape, axes)
+    rng = np.random.default_rng(case)
+    x = rng.uniform(0.7, 1.3, shape).astype(np.float32) * rng.choice([-1.0, 1.0], shape).astype(np.float32)
+    if op == "prod":
+        x = np.abs(x)
+    for keep in (False, True):
+        y = V.reduce(dev(ctx, x), axes, keep, op, init).eval(ctx).numpy()
+        y_or = O.reduce(ht(x), axes, keep, op, O.INIT_REF_ZERO if init == "ref_zero" else O.INIT_IDENTITY).numpy()
+        if op in ("max", "min"):
+            exact(y, y_or, f"{op} keep={keep}")
+        else:
+            close(y, y_or, REL_MAP, f"{op} keep={keep}")
+
+
+def test_reduce_reference_zero_accumulator(ctx):
+    """reduce.rs:282: max of an all-negative row is 0, min of an all-positive row is 0, prod is 0."""
+    say("reduce ref_zero semantics")
+    x = np.array([[-3.0, -1.0, -2.0], [4.0, 2.0, 9.0]], dtype=np.float32)
+    exact(V.max_(dev(ctx, x), 1).eval(ctx).numpy(), np.array([0.0, 9.0], np.float32), "max")
+    exact(V.min_(dev(ctx, x), 1).eval(ctx).numpy(), np.array([-3.0, 0.0], np.float32), "min")
+    exact(V.prod(dev(ctx, x), 1).eval(ctx).numpy(), np.array([-0.0, 0.0], np.float32), "prod")
+    exact(V.reduce(dev(ctx, x), 1, False, "max", "identity").eval(ctx).numpy(), np.array([-1.0, 9.0], np.float32), "true max")
+
+
+def test_reduce_strided_and_int(ctx):
+    rng = np.random.default_rng(21)
+    a = rng.standard_normal((12, 10, 8)).astype(np.float32)
+    for name in ("transpose01", "slice_mid", "permute_201"):
+        say("reduce over", name)
+        xd, xo = view_pair(ctx, a, LAYOUTS[name])
+        for axes in ([0], [1], [2], [0, 2]):
+            close(xd.sum(axes).eval(ctx).numpy(), O.rsum(xo, axes).numpy(), REL_MAP, f"{name} {axes}")
+    say("reduce int")
+    i = rng.integers(-20, 20, (9, 33)).astype(np.int32)
+    exact(dev(ctx, i).sum(1).eval(ctx).numpy(), O.rsum(ht(i), 1).numpy(), "int sum")
+    exact(dev(ctx, i).max(0).eval(ctx).numpy(), O.rmax(ht(i), 0).numpy(), "int max")
+
+
+@pytest.mark.parametrize("shape,axis", [((2, 3, 4), 1), ((64, 1000), 1), ((64, 1000), 0), ((5, 7, 300), 2), ((9, 64), 1), ((3, 1), 1)])
+@pytest.mark.parametrize("op", ["max", "min"])
+def test_reduce_arg(ctx, shape, axis, op):
+    say("reduce_arg", op, shape, axis)
+    rng = np.random.default_rng(4)
+    x = rng.integers(-6, 6, shape).astype(np.float32)  # many ties: first index must win
+    for keep in (False, True):
+        y = V.reduce_arg(dev(ctx, x), axis, keep, op).eval(ctx).numpy()
+        exact(y, O.reduce_arg(ht(x), axis, keep, op).numpy(), f"arg{op}")
+    xt_d, xt_o = view_pair(ctx, x, lambda t: t.transpose(0, 1))
+    ax = {0: 1, 1: 0}.get(axis, axis)
+    exact(V.reduce_arg(xt_d, ax, False, op).eval(ctx).numpy(), O.reduce_arg(xt_o, ax, False, op).numpy(), "transposed")
+
+
+def test_mean_var_accuracy(ctx):
+    say("mean / var / accuracy")
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((6, 50)).astype(np.float32)
+    close(dev(ctx, x).mean(1, True).eval(ctx).numpy(), O.mean(ht(x), 1, True).numpy(), REL_MAP, "mean")
+    close(dev(ctx, x).var(1, True).eval(ctx).numpy(), O.var(ht(x), 1, True).numpy(), 1e-3, "var")
+    logits = rng.standard_normal((64, 10)).astype(np.float32)
+    labels = rng.integers(0, 10, (64, 1)).astype(np.uint32)
+    acc = nn.accuracy(dev(ctx, logits), dev(ctx, labels)).eval(ctx).numpy()
+    assert float(acc[0]) == float(np.mean(np.argmax(logits, 1) == labels[:, 0]))
+
+
+# ----------------------------------------------------------------------------- indexing
+def test_gather_scatter(ctx):
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((5, 6, 7)).astype(np.float32)
+    for axis in range(3):
+        say("gather axis", axis)
+        shp = [3, 4, 5]
+        ind = rng.integers(0, x.shape[axis], shp).astype(np.uint32)
+        exact(V.gather(dev(ctx, x), dev(ctx, ind), axis).eval(ctx).numpy(), O.gather(ht(x), ht(ind), axis).numpy(), "gather")
+    say("gather embedding (stride-0 index)")
+    w = rng.standard_normal((50, 16)).astype(np.float32)
+    ids = rng.integers(0, 50, (3, 9)).astype(np.int32)
+    from sage_amd.layers import Embedding
+    emb = Embedding(50, 16)
+    emb.weight.set(S.Tensor.from_numpy(ctx, w))
+    exact(emb.pass_(dev(ctx, ids)).eval(ctx).numpy(), w[ids], "embedding")
+    exact(O.embedding(ht(w), ht(ids)).numpy(), w[ids], "oracle embedding")
+    say("gather from a transposed table")
+    xd, xo = view_pair(ctx, x, lambda t: t.transpose(0, 2))
+    ind = rng.integers(0, 7, (7, 6, 2)).astype(np.uint32)
+    exact(V.gather(xd, dev(ctx, ind), 0).eval(ctx).numpy(), O.gather(xo, ht(ind), 0).numpy(), "gather strided")
+    say("scatter, unique indices")
+    src = rng.standard_normal((4, 1)).astype(np.float32)
+    ind = rng.integers(0, 10, (4, 1)).astype(np.uint32)
+    exact(V.scatter(dev(ctx, src), dev(ctx, ind), 1, [4, 10]).eval(ctx).numpy(), O.scatter(ht(src), ht(ind), 1, [4, 10]).numpy(), "scatter")
+    say("scatter, duplicate indices (atomic sum)")
+    src = rng.standard_normal((64, 3)).astype(np.float32)
+    ind = rng.integers(0, 4, (64, 3)).astype(np.uint32)
+    want = np.zeros((4, 3), np.float64)
+    for r in range(64):
+        for c in range(3):
+            want[ind[r, c], c] += src[r, c]
+    close(V.scatter(dev(ctx, src), dev(ctx, ind), 0, [4, 3]).eval(ctx).numpy(), want, 1e-5, "scatter dup")
+
+
+def test_unslice_concat(ctx):
+    rng = np.random.default_rng(13)
+    x = rng.standard_normal((4, 3, 5)).astype(np.float32)
+    for axis, start, end in ((0, 2, 9), (1, 0, 3), (2, 1, 8)):
+        say("unslice", axis, start, end)
+        exact(V.unslice(dev(ctx, x), axis, start, end).eval(ctx).numpy(), O.unslice(ht(x), axis, start, end).numpy(), "unslice")
+    say("concat incl. a strided input")
+    a, b = rng.standard_normal((3, 2, 4)).astype(np.float32), rng.standard_normal((3, 5, 4)).astype(np.float32)
+    c = rng.standard_normal((4, 3, 4)).astype(np.float32)
+    cd, co = view_pair(ctx, c, lambda t: t.transpose(0, 1))
+    exact(V.concat([dev(ctx, a), dev(ctx, b), cd], 1).eval(ctx).numpy(), O.concat([ht(a), ht(b), co], 1).numpy(), "concat")
+
+
+# ----------------------------------------------------------------------------- GEMM
+@pytest.mark.parametrize("mkn", [(1, 1, 1), (7, 13, 5), (128, 128, 128), (130, 257, 70), (64, 49, 64), (256, 64, 96), (33, 300, 200), (1, 512, 10), (300, 1, 17)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_gemm_modes(ctx, mkn, ta, tb):
+    m, k, n = mkn
+    say("gemm", mkn, ta, tb)
+    rng = np.random.default_rng(m * 7 + n)
+    a = rng.uniform(-1, 1, (k, m) if ta else (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (n, k) if tb else (k, n)).astype(np.float32)
+    y = V.gemm(dev(ctx, a), dev(ctx, b), ta, tb).eval(ctx).numpy()
+    close(y, O.gemm(ht(a), ht(b), ta, tb).numpy(), REL_GEMM, "gemm")
+    ref64 = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+    close(y, ref64, REL_GEMM, "gemm vs float64")
+
+
+def test_gemm_offsets_and_ld(ctx):
+    """ld = strides[0] and element offsets, as gemm.rs:208-217 passes them: slices of larger matrices."""
+    say("gemm ld/offset")
+    rng = np.random.default_rng(31)
+    big_a = rng.uniform(-1, 1, (40, 90)).astype(np.float32)
+    big_b = rng.uniform(-1, 1, (100, 50)).astype(np.float32)
+    ad, ao = view_pair(ctx, big_a, lambda t: t.slice(0, 3, 36))
+    bd, bo = view_pair(ctx, big_b, lambda t: t.slice(0, 10, 100))
+    y = V.gemm(ad, bd).eval(ctx).numpy()
+    close(y, big_a[3:36].astype(np.float64) @ big_b[10:100].astype(np.float64), REL_GEMM, "row slices (offset, default strides)")
+    close(y, O.gemm(ao, bo).numpy(), REL_GEMM, "oracle")
+    # a column window has strides != default: the reference organizes (copies) it first, gemm.rs:111
+    ad, ao = view_pair(ctx, big_a, lambda t: t.slice(1, 5, 55))
+    bd, bo = view_pair(ctx, big_b, lambda t: t.slice(0, 0, 50))
+    close(V.gemm(ad, bd).eval(ctx).numpy(), O.gemm(ao, bo).numpy(), REL_GEMM, "column window")
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_gemm_batched(ctx, ta, tb):
+    say("gemm_batched", ta, tb)
+    rng = np.random.default_rng(17)
+    bt, m, k, n = 5, 37, 29, 41
+    a = rng.uniform(-1, 1, (bt, k, m) if ta else (bt, m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (bt, n, k) if tb else (bt, k, n)).astype(np.float32)
+    y = V.gemm_batched(dev(ctx, a), dev(ctx, b), ta, tb).eval(ctx).numpy()
+    close(y, O.gemm_batched(ht(a), ht(b), ta, tb).numpy(), REL_GEMM, "gemm_batched")
+
+
+def test_matmul_and_matmul_batched(ctx):
+    """matmul (gemm.rs:30-51) on rank-3 x rank-2; matmul_batched (gemm.rs:53-104) on attention layouts,
+    strided in place (fused) and through the reference's organize copies (unfused)."""
+    rng = np.random.default_rng(19)
+    x = rng.uniform(-1, 1, (3, 10, 24)).astype(np.float32)
+    w = rng.uniform(-1, 1, (24, 16)).astype(np.float32)
+    say("matmul [3,10,24] x [24,16]")
+    close(dev(ctx, x).matmul(dev(ctx, w)).eval(ctx).numpy(), O.matmul(ht(x), ht(w)).numpy(), REL_GEMM, "matmul")
+    n, l, h, d = 2, 20, 3, 8
+    q = rng.uniform(-1, 1, (n, l, h * d)).astype(np.float32)
+    k = rng.uniform(-1, 1, (n, l, h * d)).astype(np.float32)
+    for fused in (True, False):
+        V.set_fusion(fused)
+        say("attention scores, fusion", fused)
+        sep = lambda t: t.view([n, l, h, d]).transpose(2, 1)
+        s_d = sep(dev(ctx, q)).matmul_batched(sep(dev(ctx, k)).transpose(-1, -2))
+        s_o = O.matmul_batched(sep(ht(q)), sep(ht(k)).transpose(-1, -2))
+        n0 = ctx.launches
+        sd = s_d.eval(ctx).numpy()
+        if fused:
+            assert ctx.launches - n0 == 1  # no organize copies
+        close(sd, s_o.numpy(), REL_GEMM, "QK^T")
+        say("attention values + merge_heads, fusion", fused)
+        p = rng.uniform(0, 1, (n, h, l, l)).astype(np.float32)
+        av_d = dev(ctx, p).matmul_batched(sep(dev(ctx, k))).transpose(2, 1).view([n, l, h * d])
+        av_o = O.matmul_batched(ht(p), sep(ht(k))).transpose(2, 1).view([n, l, h * d])
+        n0 = ctx.launches
+        avd = av_d.eval(ctx).numpy()
+        if fused:
+            assert ctx.launches - n0 == 1  # result written in merged layout, no copy
+        close(avd, av_o.numpy(), REL_GEMM, "PV merged")
+
+
+def test_gemm_epilogues(ctx):
+    """Dense (+bias), Dense+ReLU, Dense+GELU, Dense+bias+residual, relu(conv+bias+x), scores/8."""
+    rng = np.random.default_rng(23)
+    x = rng.standard_normal((6, 11, 40)).astype(np.float32)
+    w = (rng.standard_normal((40, 24)) * 0.2).astype(np.float32)
+    b = rng.standard_normal((24,)).astype(np.float32)
+    r = rng.standard_normal((6, 11, 24)).astype(np.float32)
+    cases = {
+        "bias": (lambda X, W, Bi, R: X.matmul(W) + Bi, lambda X, W, Bi, R: O.dense(X, W, Bi)),
+        "bias_relu": (lambda X, W, Bi, R: nn.relu(X.matmul(W) + Bi), lambda X, W, Bi, R: O.relu(O.dense(X, W, Bi))),
+        "bias_gelu": (lambda X, W, Bi, R: nn.gelu(X.matmul(W) + Bi),
+                      lambda X, W, Bi, R: O.binary("mul", O.binary("mul", O.dense(X, W, Bi), 0.5),
+                                                   O.binary("add", O.unary("erf", O.binary("div", O.dense(X, W, Bi), float(np.sqrt(np.float32(2))))), 1.0))),
+        "bias_res": (lambda X, W, Bi, R: (X.matmul(W) + Bi) + R, lambda X, W, Bi, R: O.binary("add", O.dense(X, W, Bi), R)),
+        "res_first": (lambda X, W, Bi, R: R + (X.matmul(W) + Bi), lambda X, W, Bi, R: O.binary("add", R, O.dense(X, W, Bi))),
+        "relu_bias_res": (lambda X, W, Bi, R: nn.relu((X.matmul(W) + Bi) + R), lambda X, W, Bi, R: O.relu(O.binary("add", O.dense(X, W, Bi), R))),
+        "scale": (lambda X, W, Bi, R: X.matmul(W) / 8.0, lambda X, W, Bi, R: O.binary("div", O.matmul(X, W), 8.0)),
+    }
+    for name, (fd, fo) in cases.items():
+        say("epilogue", name)
+        n0 = ctx.launches
+        y = fd(dev(ctx, x), dev(ctx, w), dev(ctx, b), dev(ctx, r)).eval(ctx).numpy()
+        assert ctx.launches - n0 == 1, f"{name}: expected one fused GEMM launch, got {ctx.launches - n0}"
+        close(y, fo(ht(x), ht(w), ht(b), ht(r)).numpy(), REL_GEMM, name)
+        V.set_fusion(False)
+        yu = fd(dev(ctx, x), dev(ctx, w), dev(ctx, b), dev(ctx, r)).eval(ctx).numpy()
+        V.set_fusion(True)
+        close(y, yu, REL_GEMM, name + " vs unfused")
+    say("shared GEMM output is not folded twice")
+    X, W, Bi = dev(ctx, x), dev(ctx, w), dev(ctx, b)
+    g = X.matmul(W)
+    y1, y2 = S.evaluate(ctx, [g + Bi, g * 2.0])
+    close(y2.numpy(), 2.0 * (y1.numpy() - b), REL_GEMM, "shared")
+
+
+# ----------------------------------------------------------------------------- conv
+IM2COL_CASES = [
+    ((2, 28, 28, 1), 7, 2, 3, 1), ((2, 14, 14, 64), 3, 2, 1, 1), ((3, 7, 7, 64), 3, 1, 1, 1), ((2, 7, 7, 64), 1, 2, 0, 1),
+    ((1, 5, 4, 3), [3, 2], 1, 0, 1), ((2, 9, 11, 6), [2, 3], [2, 1], [1, 2], [2, 1]), ((2, 1, 1, 512), 1, 1, 0, 1),
+]
+
+
+@pytest.mark.parametrize("case", range(len(IM2COL_CASES)))
+def test_im2col(ctx, case):
+    shape, ker, stride, pad, dil = IM2COL_CASES[case]
+    say("im2col", shape, ker, stride, pad, dil)
+    x = np.random.default_rng(case).standard_normal(shape).astype(np.float32)
+    exact(V.im2col(dev(ctx, x), ker, stride, pad, dil).eval(ctx).numpy(), O.im2col(ht(x), ker, stride, pad, dil).numpy(), "im2col")
+
+
+def test_conv_and_pools(ctx):
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(29)
+    x = rng.standard_normal((2, 12, 10, 5)).astype(np.float32)
+    f = (rng.standard_normal((3, 3, 5, 7)) * 0.3).astype(np.float32)
+    b = rng.standard_normal((7,)).astype(np.float32)
+    say("conv2d vs oracle and torch")
+    from sage_amd.layers import Conv2d
+    conv = Conv2d(5, 7, 3, 2, 1, 1)
+    conv.weight.set(S.Tensor.from_numpy(ctx, f))
+    conv.bias.set(S.Tensor.from_numpy(ctx, b))
+    y = conv.pass_(dev(ctx, x)).eval(ctx).numpy()
+    close(y, O.conv2d_layer(ht(x), ht(f), ht(b), 2, 1).numpy(), REL_GEMM, "conv oracle")
+    t = F.conv2d(torch.from_numpy(x).permute(0, 3, 1, 2).double(), torch.from_numpy(f).permute(3, 2, 0, 1).double(),
+                 torch.from_numpy(b).double(), stride=2, padding=1).permute(0, 2, 3, 1).numpy()
+    close(y, t, REL_GEMM, "conv torch")
+    say("max / avg pool")
+    xp = np.abs(x)
+    exact(V.max_pool_2d(dev(ctx, xp), 3, 2, 1, 1).eval(ctx).numpy(), O.max_pool_2d(ht(xp), 3, 2, 1, 1).numpy(), "max_pool")
+    close(V.avg_pool_2d(dev(ctx, xp), 2, 2, 0, 1).eval(ctx).numpy(), O.avg_pool_2d(ht(xp), 2, 2, 0, 1).numpy(), REL_MAP, "avg_pool")
+
+
+# ----------------------------------------------------------------------------- fused row operators
+@pytest.mark.parametrize("shape", [(64, 128), (5, 1000), (3, 4, 16, 16), (9, 1024), (2, 2052), (7, 10)])
+def test_softmax_fused_vs_composed_vs_oracle(ctx, shape):
+    say("softmax", shape)
+    rng = np.random.default_rng(len(shape))
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    x[0] -= 20.0  # an all-negative row: the reference's zero-initialised max shows here
+    ax = len(shape) - 1
+    yf = nn.softmax(dev(ctx, x), ax).eval(ctx).numpy()
+    V.set_fusion(False)
+    yc = nn.softmax(dev(ctx, x), ax).eval(ctx).numpy()
+    yo = O.softmax(ht(x), ax).numpy()
+    close(yf, yo, REL_MAP, "fused vs oracle")
+    close(yc, yo, REL_MAP, "composed vs oracle")
+    close(yf.sum(-1), np.ones(shape[:-1]), 1e-5, "rows sum to 1")
+
+
+def test_softmax_with_mask_addend(ctx):
+    say("softmax(scores/8 + mask)")
+    rng = np.random.default_rng(41)
+    n, h, l = 3, 2, 32
+    s = rng.standard_normal((n, h, l, l)).astype(np.float32) * 4
+    m = (rng.uniform(0, 1, (n, l)) > 0.3).astype(np.float32)
+    m[:, 0] = 1.0
+
+    def dev_expr():
+        md = (-dev(ctx, m).view([n, 1, 1, l]) + 1.0) * -1e5
+        return nn.softmax(dev(ctx, s) / 8.0 + md, 3)
+
+    mo = O.binary("mul", O.binary("add", O.unary("neg", ht(m).view([n, 1, 1, l])), 1.0), -1e5)
+    yo = O.softmax(O.binary("add", O.binary("div", ht(s), 8.0), mo), 3).numpy()
+    close(dev_expr().eval(ctx).numpy(), yo, REL_MAP, "fused")
+    V.set_fusion(False)
+    close(dev_expr().eval(ctx).numpy(), yo, REL_MAP, "composed")
+
+
+@pytest.mark.parametrize("shape", [(5, 10), (512, 1024), (37, 1000), (16, 4096)])
+def test_softmax_cross_entropy(ctx, shape):
+    say("softmax_cross_entropy", shape)
+    rng = np.random.default_rng(shape[0])
+    x = rng.standard_normal(shape).astype(np.float32)
+    lab = rng.integers(0, shape[1], (shape[0], 1)).astype(np.int32)
+    yf = nn.softmax_cross_entropy(dev(ctx, x), dev(ctx, lab)).eval(ctx).numpy()
+    V.set_fusion(False)
+    yc = nn.softmax_cross_entropy(dev(ctx, x), dev(ctx, lab)).eval(ctx).numpy()
+    yo = O.softmax_cross_entropy(ht(x), ht(lab.view(np.uint32).astype(np.uint32))).numpy()
+    x64 = x.astype(np.float64)
+    ref = -(x64[np.arange(shape[0]), lab[:, 0]] - np.log(np.exp(x64).sum(1)))
+    for name, y in (("fused", yf), ("composed", yc), ("oracle", yo)):
+        close(y, ref, REL_MAP, name + " vs float64")
+    close(yf, yo, REL_MAP, "fused vs oracle")
+
+
+@pytest.mark.parametrize("shape,per_feature", [((8, 16, 768), False), ((8, 16, 768), True), ((5, 100), False), ((3, 2050), True), ((64, 64), True)])
+def test_layer_norm(ctx, shape, per_feature):
+    say("layer_norm", shape, per_feature)
+    rng = np.random.default_rng(shape[-1])
+    x = (rng.standard_normal(shape) * 2 + 0.5).astype(np.float32)
+    n = shape[-1] if per_feature else 1
+    g = rng.uniform(0.5, 1.5, (n,)).astype(np.float32)
+    b = rng.standard_normal((n,)).astype(np.float32)
+    ax = len(shape) - 1
+    yf = nn.layer_norm(dev(ctx, x), ax, dev(ctx, g), dev(ctx, b), 1e-5).eval(ctx).numpy()
+    V.set_fusion(False)
+    yc = nn.layer_norm(dev(ctx, x), ax, dev(ctx, g), dev(ctx, b), 1e-5).eval(ctx).numpy()
+    yo = O.layer_norm(ht(x), ax, ht(g), ht(b), 1e-5).numpy()
+    x64 = x.astype(np.float64)
+    ref = (x64 - x64.mean(-1, keepdims=True)) / np.sqrt(x64.var(-1, keepdims=True) + 1e-5) * g + b
+    close(yf, ref, 5e-4, "fused vs float64")
+    close(yc, ref, 5e-4, "composed vs float64")
+    close(yo, ref, 5e-4, "oracle vs float64")
+    close(yf, yo, 5e-4, "fused vs oracle")

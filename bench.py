@@ -1,0 +1,209 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X: BERT-base forward (b32, s128, fp32) through the C ABI.
+
+A step is one full forward pass (embedding gathers + LayerNorm, 12 encoder layers, classifier) over
+one synthetic batch that is already resident in HBM.  The model is the configuration the metric is
+quoted on — erf-GELU, LayerNorm eps 1e-12 with per-feature gamma/beta, weights ~N(0, 0.02) — built
+from the same operators the parity tests check; `--variant reference` runs the composition the
+reference's own models/bert.rs builds instead (ReLU, eps 1e-5, scalar gamma = beta).
+
+Prints ONE JSON line: whole-job throughput, the roofline of the dominant kernel (the fp32 MFMA
+GEMM instantiation that takes the most time, timed per launch with HIP events on the stream it
+runs on, inside the timed steps) and the CPU oracle timed on a bounded sample of the same workload.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def build_bert(ctx, variant, batch, seq, layers, rng):
+    import sage_amd as S
+    from sage_amd.bert import Bert, BertConfig
+    cfg = BertConfig.base()
+    cfg.num_layers = layers
+    exact = variant == "reference"
+    model = Bert(cfg, reference_exact=exact, segments=0)
+    for p in model.params():
+        n = p.label or ""
+        if "layer_norm.gamma" in n:
+            a = np.ones(p.extents, np.float32)
+        elif "layer_norm.beta" in n:
+            a = np.ones(p.extents, np.float32) if exact else np.zeros(p.extents, np.float32)
+        elif n.endswith(".bias"):
+            a = np.zeros(p.extents, np.float32)
+        else:
+            a = (rng.standard_normal(p.extents) * 0.02).astype(np.float32)
+        p.set(S.Tensor.from_numpy(ctx, a))
+    ids = rng.integers(0, cfg.num_vocabs, (batch, seq)).astype(np.int32)
+    mask = np.ones((batch, seq), np.float32)
+    ids_v = S.Var.new(S.Tensor.from_numpy(ctx, ids))
+    mask_v = S.Var.new(S.Tensor.from_numpy(ctx, mask))
+    logits = model.pass_(ids_v, mask_v, ctx)
+    return cfg, model, logits
+
+
+def gemm_calls(ctx, prog):
+    """(call index, kernel name, flops) for every GEMM launch of the compiled program."""
+    from sage_amd import abi
+    lib = abi.lib()
+    out = []
+    for i, (fn, args, _) in enumerate(prog.calls):
+        if fn in (lib.sg_gemm, lib.sg_gemm_batched, lib.sg_matmul_strided):
+            if fn is lib.sg_matmul_strided:
+                a, b, c = (x._obj for x in args[:3])
+                ta = tb = 0
+            else:
+                ta, tb = args[0], args[1]
+                a, b, c = (x._obj for x in args[2:5])
+            r = c.rank
+            M, N = c.extents[r - 2], c.extents[r - 1]
+            if fn is lib.sg_matmul_strided:
+                K = a.extents[r - 1]
+                a_kc = a.strides[r - 1] == 1
+                b_nc = b.strides[r - 1] == 1
+            else:
+                K = a.extents[r - 2] if ta else a.extents[r - 1]
+                a_kc, b_nc = not ta, not tb
+            batch = 1
+            for d in range(r - 2):
+                batch *= c.extents[d]
+            buf = C.create_string_buffer(128)
+            ctx.check(lib.sg_gemm_kernel_name(ctx.handle, M, N, K, batch, int(a_kc), int(b_nc), buf, 128))
+            out.append((i, buf.value.decode(), 2.0 * M * N * K * batch + M * N * batch, (M, N, K, batch)))
+    return out
+
+
+def run_timed(ctx, prog, timed):
+    """One replay of the program with a HIP event pair around each call index in `timed`."""
+    from sage_amd import abi
+    lib = abi.lib()
+    h = ctx.handle
+    for i, (fn, args, _) in enumerate(prog.calls):
+        if i in timed:
+            a, b = timed[i]
+            lib.sg_event_record(h, a)
+            rc = fn(h, *args)
+            lib.sg_event_record(h, b)
+        else:
+            rc = fn(h, *args)
+        if rc:
+            ctx.check(rc)
+
+
+def cpu_baseline(variant, batch, seq, rng_seed):
+    """The CPU oracle (oracle/: C restatement of the reference kernels, OpenMP over work-items) on one
+    of the 12 encoder layers at the full b32 x s128 shape; the layer time x 12 gives seqs/s."""
+    from oracle import oracle as O
+    rng = np.random.default_rng(rng_seed)
+    e, hdim, heads = 768, 3072, 12
+    w = lambda i, o: O.HT.from_numpy((rng.standard_normal((i, o)) * 0.02).astype(np.float32))
+    z = lambda n: O.HT.from_numpy(np.zeros(n, np.float32))
+    nln = 1 if variant == "reference" else e
+    one = lambda: O.HT.from_numpy(np.ones(nln, np.float32))
+    p = {"wq": w(e, e), "bq": z(e), "wk": w(e, e), "bk": z(e), "wv": w(e, e), "bv": z(e), "wo": w(e, e), "bo": z(e),
+         "ln1_g": one(), "ln1_b": z(nln), "w1": w(e, hdim), "b1": z(hdim), "w2": w(hdim, e), "b2": z(e), "ln2_g": one(), "ln2_b": z(nln)}
+    x = O.HT.from_numpy(rng.standard_normal((batch, seq, e)).astype(np.float32))
+    mask = O.HT.from_numpy(np.ones((batch, seq), np.float32))
+    act, eps = ("relu", 1e-5) if variant == "reference" else ("gelu", 1e-12)
+    t0 = time.perf_counter()
+    O.bert_layer(x, mask, p, heads, act, eps)
+    dt = time.perf_counter() - t0
+    return {"value": batch / (12.0 * dt), "unit": "seqs/s", "cores": O.num_threads(), "kind": "port",
+            "sample": f"1 of 12 encoder layers at b{batch} s{seq} in {dt:.2f} s, x12 (embedding and classifier left out)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--variant", choices=["config", "reference"], default="config")
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--seq", type=int, default=128)
+    ap.add_argument("--layers", type=int, default=12)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: every box in this run has one MI355X and the hot path uses no "
+              "collectives; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import sage_amd as S
+    from sage_amd import abi
+    lib = abi.lib()
+    ctx = S.Context(0)
+    rng = np.random.default_rng(5)
+    cfg, model, logits = build_bert(ctx, a.variant, a.batch, a.seq, a.layers, rng)
+    prog = S.Program(ctx, [logits])  # first evaluation: builds kernels, allocates every buffer
+    ctx.sync()
+    out0 = prog.outputs[0].numpy()
+    if not np.all(np.isfinite(out0)):
+        raise SystemExit("non-finite model output")
+
+    # the dominant kernel: the GEMM instantiation with the most flops in the program
+    gc = gemm_calls(ctx, prog)
+    by_name = {}
+    for i, name, flops, shape in gc:
+        by_name.setdefault(name, []).append((i, flops, shape))
+    dom = max(by_name, key=lambda n: sum(f for _, f, _ in by_name[n]))
+    def new_event():
+        e = C.c_void_p()
+        ctx.check(lib.sg_event_create(ctx.handle, C.byref(e)))
+        return e
+
+    # one event pair per (step, launch of the dominant kernel); all are read after the timed region
+    pairs = [{i: (new_event(), new_event()) for i, _, _ in by_name[dom]} for _ in range(a.steps)]
+
+    for _ in range(a.warmup):
+        prog.run()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for step in range(a.steps):
+        run_timed(ctx, prog, pairs[step])
+    ctx.sync()
+    dt = time.perf_counter() - t0
+    kernel_ms = []
+    for step in range(a.steps):
+        for i, (e0, e1) in pairs[step].items():
+            ms = C.c_float()
+            ctx.check(lib.sg_event_elapsed_ms(ctx.handle, e0, e1, C.byref(ms)))
+            kernel_ms.append(ms.value)
+    ms_per_step = dt / a.steps * 1e3
+
+    flops_per_launch = float(np.mean([f for _, f, _ in by_name[dom]]))
+    avg_ms = float(np.mean(kernel_ms))
+    achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
+    total_gemm_flops = sum(f for _, _, f, _ in gc)
+    res = {
+        "metric": "BERT-base fwd seqs/sec (b32,s128,fp32)",
+        "value": a.batch / (ms_per_step * 1e-3),
+        "unit": "seqs/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"bert_base_forward_b{a.batch}_s{a.seq}_fp32", "variant": a.variant, "layers": a.layers,
+                   "hidden": cfg.embed_dim, "heads": cfg.num_attention_heads, "ffn": cfg.hidden_dim, "vocab": cfg.num_vocabs,
+                   "launches_per_step": len(prog.calls), "gemm_tflops_whole_step": total_gemm_flops / (ms_per_step * 1e-3) / 1e12},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None, "kernel": dom,
+                     "launches_per_step": len(by_name[dom]), "avg_launch_ms": avg_ms, "flops_per_launch": flops_per_launch,
+                     "shapes_mnkb": sorted({s for _, _, s in by_name[dom]})},
+    }
+    if not a.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(a.variant, a.batch, a.seq, 6)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

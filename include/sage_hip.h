@@ -98,6 +98,14 @@ int sg_fill_u32(sg_ctx *ctx, void *dst_dev, uint32_t pattern, uint64_t count);
 int sg_sync(sg_ctx *ctx);
 void *sg_stream(sg_ctx *ctx);
 
+/* Device-side timing on the context's stream.  The reference only wall-clocks a routine on the
+ * host (Routine::exec, session.rs:619, 667-668); these wrap hipEvent so a caller can time the
+ * launches it issued between two records. */
+int sg_event_create(sg_ctx *ctx, void **event);
+int sg_event_record(sg_ctx *ctx, void *event);
+int sg_event_elapsed_ms(sg_ctx *ctx, void *start, void *stop, float *ms);
+int sg_event_destroy(sg_ctx *ctx, void *event);
+
 const char *sg_last_error(sg_ctx *ctx);
 int sg_last_oom(sg_ctx *ctx, uint64_t *needed, uint64_t *total);
 /* Number of distinct kernels built at run time so far (Context::kernels, context.rs:29-31). */
@@ -217,6 +225,12 @@ int sg_gemm_batched(sg_ctx *ctx, int transpose_a, int transpose_b, const sg_tens
  * permuted attention heads (bert.rs:282-302) are consumed and produced in place. */
 int sg_matmul_strided(sg_ctx *ctx, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c,
                       const sg_gemm_epilogue *epi);
+
+/* Name of the kernel instantiation a GEMM of this shape is dispatched to (tile sizes and operand
+ * layouts are template arguments), as it appears in a rocprofv3 kernel trace.  The reference has one
+ * fixed 8x8 kernel per transpose mode (gemm.rs:208-221); here the tile is chosen per shape. */
+int sg_gemm_kernel_name(sg_ctx *ctx, int64_t M, int64_t N, int64_t K, int64_t batch, int a_k_contiguous,
+                        int b_n_contiguous, char *buf, uint64_t cap);
 
 /* ---- convolution feeder: ops/conv.rs --------------------------------------------------------- */
 

@@ -4,4 +4,4 @@ include/sage_hip.h.  All compute runs in sage_amd/libsage_hip.so; there is no CP
 from . import abi, bert, layers, nn, resnet, var  # noqa: F401
 from .shape import Shape  # noqa: F401
 from .tensor import FLOAT, INT, UINT, Context, Tensor  # noqa: F401
-from .var import Var, evaluate, set_fusion  # noqa: F401
+from .var import Program, Var, evaluate, set_fusion  # noqa: F401

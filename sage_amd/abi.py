@@ -64,6 +64,10 @@ PROTOTYPES = {
     "sg_fill_u32": (C.c_int, [_CTX, C.c_void_p, C.c_uint32, C.c_uint64]),
     "sg_sync": (C.c_int, [_CTX]),
     "sg_stream": (C.c_void_p, [_CTX]),
+    "sg_event_create": (C.c_int, [_CTX, C.POINTER(C.c_void_p)]),
+    "sg_event_record": (C.c_int, [_CTX, C.c_void_p]),
+    "sg_event_elapsed_ms": (C.c_int, [_CTX, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
+    "sg_event_destroy": (C.c_int, [_CTX, C.c_void_p]),
     "sg_last_error": (C.c_char_p, [_CTX]),
     "sg_last_oom": (C.c_int, [_CTX, _U64P, _U64P]),
     "sg_kernel_cache_size": (C.c_int, [_CTX]),
@@ -79,6 +83,7 @@ PROTOTYPES = {
     "sg_gemm": (C.c_int, [_CTX, C.c_int, C.c_int, _TP, _TP, _TP, C.POINTER(sg_gemm_epilogue)]),
     "sg_gemm_batched": (C.c_int, [_CTX, C.c_int, C.c_int, _TP, _TP, _TP, C.POINTER(sg_gemm_epilogue)]),
     "sg_matmul_strided": (C.c_int, [_CTX, _TP, _TP, _TP, C.POINTER(sg_gemm_epilogue)]),
+    "sg_gemm_kernel_name": (C.c_int, [_CTX, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_char_p, C.c_uint64]),
     "sg_im2col": (C.c_int, [_CTX, _TP, _TP, _I32P, _I32P, _I32P, _I32P]),
     "sg_softmax_lastaxis": (C.c_int, [_CTX, _TP, _TP, _TP]),
     "sg_softmax_cross_entropy": (C.c_int, [_CTX, _TP, _TP, _TP]),

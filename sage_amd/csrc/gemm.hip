@@ -230,19 +230,20 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
 
 // Tile choice: the largest tile that still gives every CU at least one workgroup, preferring an
 // exact multiple of the CU count (no partially filled last round of workgroups).
-int launch_gemm(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
-    struct Cfg { int bm, bn; };
-    static const Cfg cfgs[] = {{128, 128}, {128, 96}, {128, 64}, {64, 64}};
-    const int64_t cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+struct TileCfg { int bm, bn, waves_m; };
+const TileCfg kTileCfgs[] = {{128, 128, 2}, {128, 96, 4}, {128, 64, 2}, {64, 64, 2}};
+
+int choose_tile(int num_cus, int M, int N, int batch) {
+    const int64_t cus = num_cus > 0 ? num_cus : 256;
     int best = 3;
     double best_score = -1.0;
     for (int c = 0; c < 4; ++c) {
-        const int64_t tm = (p.M + cfgs[c].bm - 1) / cfgs[c].bm, tn = (p.N + cfgs[c].bn - 1) / cfgs[c].bn;
+        const int64_t tm = (M + kTileCfgs[c].bm - 1) / kTileCfgs[c].bm, tn = (N + kTileCfgs[c].bn - 1) / kTileCfgs[c].bn;
         const int64_t tiles = tm * tn * batch;
         const int64_t rounds = (tiles + cus - 1) / cus;
         // useful work / (rounds * cus * tile area): fill of the last round and of edge tiles
-        const double useful = (double)p.M * p.N * batch;
-        const double spent = (double)rounds * cus * cfgs[c].bm * cfgs[c].bn;
+        const double useful = (double)M * N * batch;
+        const double spent = (double)rounds * cus * kTileCfgs[c].bm * kTileCfgs[c].bn;
         double score = useful / spent;
         // larger tiles re-read less of A and B: small bonus
         score *= 1.0 + 0.05 * (3 - c);
@@ -253,7 +254,11 @@ int launch_gemm(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
     }
     const char *force = getenv("SAGE_GEMM_TILE");
     if (force && force[0] >= '0' && force[0] <= '3') best = force[0] - '0';
-    switch (best) {
+    return best;
+}
+
+int launch_gemm(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
+    switch (choose_tile(ctx->num_cus, p.M, p.N, batch)) {
     case 0: return launch_cfg<128, 128, 2>(ctx, p, batch, a_kc, b_nc);
     case 1: return launch_cfg<128, 96, 4>(ctx, p, batch, a_kc, b_nc);
     case 2: return launch_cfg<128, 64, 2>(ctx, p, batch, a_kc, b_nc);
@@ -342,6 +347,16 @@ int check_f32(sg_ctx *ctx, const sg_tensor *a, const sg_tensor *b, const sg_tens
 }
 
 }  // namespace
+
+extern "C" int sg_gemm_kernel_name(sg_ctx *ctx, int64_t M, int64_t N, int64_t K, int64_t batch, int a_k_contiguous,
+                                   int b_n_contiguous, char *buf, uint64_t cap) {
+    if (!ctx || !buf || cap < 8) return SG_ERR_ARG;
+    (void)K;
+    const TileCfg &t = kTileCfgs[choose_tile(ctx->num_cus, (int)M, (int)N, (int)batch)];
+    snprintf(buf, cap, "gemm_mfma_kernel<%d, %d, %d, %s, %s>", t.bm, t.bn, t.waves_m, a_k_contiguous ? "true" : "false",
+             b_n_contiguous ? "true" : "false");
+    return SG_OK;
+}
 
 extern "C" int sg_gemm(sg_ctx *ctx, int ta, int tb, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c,
                        const sg_gemm_epilogue *epi) {

@@ -189,6 +189,33 @@ int sg_sync(sg_ctx *ctx) {
 
 void *sg_stream(sg_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
 
+int sg_event_create(sg_ctx *ctx, void **event) {
+    if (!ctx || !event) return SG_ERR_ARG;
+    hipEvent_t e;
+    SG_HIP(ctx, hipEventCreate(&e));
+    *event = (void *)e;
+    return SG_OK;
+}
+
+int sg_event_record(sg_ctx *ctx, void *event) {
+    if (!ctx || !event) return SG_ERR_ARG;
+    SG_HIP(ctx, hipEventRecord((hipEvent_t)event, ctx->stream));
+    return SG_OK;
+}
+
+int sg_event_elapsed_ms(sg_ctx *ctx, void *start, void *stop, float *ms) {
+    if (!ctx || !start || !stop || !ms) return SG_ERR_ARG;
+    SG_HIP(ctx, hipEventSynchronize((hipEvent_t)stop));
+    SG_HIP(ctx, hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return SG_OK;
+}
+
+int sg_event_destroy(sg_ctx *ctx, void *event) {
+    if (!ctx || !event) return SG_ERR_ARG;
+    SG_HIP(ctx, hipEventDestroy((hipEvent_t)event));
+    return SG_OK;
+}
+
 const char *sg_last_error(sg_ctx *ctx) { return ctx ? ctx->last_error.c_str() : "null context"; }
 
 int sg_last_oom(sg_ctx *ctx, uint64_t *needed, uint64_t *total) {

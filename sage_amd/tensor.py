@@ -108,6 +108,15 @@ class Tensor:
         sh = Shape(extents)
         return Tensor(Buffer(ctx, max(1, sh.size()) * 4), dtype, sh)
 
+    def copy_from_numpy(self, a):
+        """Overwrite this (dense) tensor's elements with `a` (Buffer::write, device.rs:111-128)."""
+        ctx = self.buf.ctx
+        a = np.ascontiguousarray(np.asarray(a, dtype=_NP_OF[self.dtype]))
+        if list(a.shape) != self.shape.extents or not self.is_dense():
+            raise abi.ShapeError(abi.ERR_SHAPE, "copy_from_numpy needs a dense tensor of the same extents")
+        dst = C.c_void_p(self.buf.ptr + self.shape.offset * 4)
+        ctx.check(ctx._lib.sg_memcpy_h2d(ctx.handle, dst, a.ctypes.data_as(C.c_void_p), a.nbytes))
+
     def numpy(self):
         """Blocking read of the whole buffer, then the strided view is taken on the host."""
         ctx = self.buf.ctx

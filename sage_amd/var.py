@@ -592,8 +592,31 @@ def evaluate(ctx, targets):
     return out
 
 
-class _Evaluator:
+class Program:
+    """Program::compile / Program::exec (session.rs:62-206, 208-468) for a fixed graph: the first
+    evaluation decides every launch (fusion, epilogues, layouts) and allocates every intermediate;
+    `run()` replays exactly those launches on the same buffers, so a repeated forward pass costs no
+    graph walking and no allocation.  New input values are supplied by writing into the data
+    tensors the graph was built on (`Tensor.copy_from_numpy`)."""
+
     def __init__(self, ctx, targets):
+        self.ctx = ctx
+        self.calls = []
+        self._ev = _Evaluator(ctx, targets, record=self.calls)
+        self.outputs = [self._ev.get(t) for t in targets]
+
+    def run(self):
+        h, check = self.ctx.handle, self.ctx.check
+        for fn, args, _ in self.calls:
+            rc = fn(h, *args)
+            if rc:
+                check(rc)
+        self.ctx.launches += len(self.calls)
+        return self.outputs
+
+
+class _Evaluator:
+    def __init__(self, ctx, targets, record=None):
         self.ctx = ctx
         self.lib = ctx._lib
         self.memo = {}
@@ -612,6 +635,8 @@ class _Evaluator:
                 self.users.setdefault(id(i), []).append(v)
                 stack.append(i)
         self.keep = {}  # id -> Var, keeps nodes alive while ids are used as keys
+        self.record = record
+        self.keepalive = []
 
     # ---- helpers
     def n_users(self, v):
@@ -632,9 +657,14 @@ class _Evaluator:
             self.keep[id(v)] = v
         return t
 
-    def launch(self, rc):
+    def call(self, fn, *args):
+        """Issue one operator launch through the C ABI; remember it when a Program is being compiled.
+        The epilogue struct keeps pointers into `keepalive` objects, so those are stored too."""
         self.ctx.launches += 1
-        self.ctx.check(rc)
+        self.ctx.check(fn(self.ctx.handle, *args))
+        if self.record is not None:
+            self.record.append((fn, args, list(self.keepalive)))
+        self.keepalive = []
 
     def out(self, extents, dtype):
         return Tensor.uninit(self.ctx, extents, dtype)
@@ -722,7 +752,7 @@ class _Evaluator:
             arr[i].kind, arr[i].op, arr[i].dtype, arr[i].bits = k, o, d, b
         ins = (abi.sg_tensor * max(1, len(leaves)))(*[t.c() for t in leaves])
         yc = y.c()
-        self.launch(self.lib.sg_map(self.ctx.handle, arr, n, ins, len(leaves), C.byref(yc)))
+        self.call(self.lib.sg_map, arr, n, ins, len(leaves), C.byref(yc))
         return y
 
     def run_copy(self, x):
@@ -753,7 +783,7 @@ class _Evaluator:
         op = {"sum": abi.R_SUM, "prod": abi.R_PROD, "max": abi.R_MAX, "min": abi.R_MIN}[v.attrs["op"]]
         init = abi.INIT_REF_ZERO if v.attrs["init"] == "ref_zero" else abi.INIT_IDENTITY
         xc, yc = x.c(), y.c()
-        self.launch(self.lib.sg_reduce(self.ctx.handle, op, ax, len(axes), init, C.byref(xc), C.byref(yc)))
+        self.call(self.lib.sg_reduce, op, ax, len(axes), init, C.byref(xc), C.byref(yc))
         return y
 
     def _ev_reduce_arg(self, v):
@@ -761,28 +791,28 @@ class _Evaluator:
         y = self.out(v.extents, UINT)
         xc, yc = x.c(), y.c()
         op = abi.RA_MAX if v.attrs["op"] == "max" else abi.RA_MIN
-        self.launch(self.lib.sg_reduce_arg(self.ctx.handle, op, v.attrs["axis"], C.byref(xc), C.byref(yc)))
+        self.call(self.lib.sg_reduce_arg, op, v.attrs["axis"], C.byref(xc), C.byref(yc))
         return y
 
     def _ev_gather(self, v):
         x, ind = self.get(v.inputs[0]), self.get(v.inputs[1])
         y = self.out(v.extents, v.dtype)
         xc, ic, yc = x.c(), ind.c(), y.c()
-        self.launch(self.lib.sg_gather(self.ctx.handle, v.attrs["axis"], C.byref(xc), C.byref(ic), C.byref(yc)))
+        self.call(self.lib.sg_gather, v.attrs["axis"], C.byref(xc), C.byref(ic), C.byref(yc))
         return y
 
     def _ev_scatter(self, v):
         x, ind = self.get(v.inputs[0]), self.get(v.inputs[1])
         y = self.out(v.extents, v.dtype)
         xc, ic, yc = x.c(), ind.c(), y.c()
-        self.launch(self.lib.sg_scatter(self.ctx.handle, v.attrs["axis"], C.byref(xc), C.byref(ic), C.byref(yc)))
+        self.call(self.lib.sg_scatter, v.attrs["axis"], C.byref(xc), C.byref(ic), C.byref(yc))
         return y
 
     def _ev_unslice(self, v):
         x = self.get(v.inputs[0])
         y = self.out(v.extents, v.dtype)
         xc, yc = x.c(), y.c()
-        self.launch(self.lib.sg_unslice(self.ctx.handle, v.attrs["axis"], v.attrs["start"], C.byref(xc), C.byref(yc)))
+        self.call(self.lib.sg_unslice, v.attrs["axis"], v.attrs["start"], C.byref(xc), C.byref(yc))
         return y
 
     def _ev_concat(self, v):
@@ -790,7 +820,7 @@ class _Evaluator:
         y = self.out(v.extents, v.dtype)
         ins = (abi.sg_tensor * len(xs))(*[t.c() for t in xs])
         yc = y.c()
-        self.launch(self.lib.sg_concat(self.ctx.handle, v.attrs["axis"], ins, len(xs), C.byref(yc)))
+        self.call(self.lib.sg_concat, v.attrs["axis"], ins, len(xs), C.byref(yc))
         return y
 
     def _ev_im2col(self, v):
@@ -801,7 +831,7 @@ class _Evaluator:
         a = v.attrs
         arr = lambda p: (C.c_int32 * 2)(*p)
         xc, yc = x.c(), y.c()
-        self.launch(self.lib.sg_im2col(self.ctx.handle, C.byref(xc), C.byref(yc), arr(a["ker"]), arr(a["stride"]), arr(a["pad"]), arr(a["dil"])))
+        self.call(self.lib.sg_im2col, C.byref(xc), C.byref(yc), arr(a["ker"]), arr(a["stride"]), arr(a["pad"]), arr(a["dil"]))
         return y
 
     # ---- GEMM family, with optional epilogue and destination layout
@@ -826,8 +856,10 @@ class _Evaluator:
         """Run gemm / gemm_batched / matmul_nd node `g`.  `dest`: a Tensor view with g's extents to
         write into (any batch strides, unit last stride); default a fresh dense tensor."""
         a, b = self.get(g.inputs[0]), self.get(g.inputs[1])
-        keep = []
+        keep = self.keepalive
         e = self._epi_struct(epi, keep)
+        if e is not None:
+            keep.append(e)
         ep = C.byref(e) if e is not None else None
         y = dest if dest is not None else self.out(g.extents, FLOAT)
         if g.op == "matmul_nd":
@@ -839,7 +871,7 @@ class _Evaluator:
             if not usable(b):
                 b = self.run_copy(b)
             ac, bc, yc = a.c(), b.c(), y.c()
-            self.launch(self.lib.sg_matmul_strided(self.ctx.handle, C.byref(ac), C.byref(bc), C.byref(yc), ep))
+            self.call(self.lib.sg_matmul_strided, C.byref(ac), C.byref(bc), C.byref(yc), ep)
             return y
         if not a.is_dense():
             a = self.run_copy(a)
@@ -847,7 +879,7 @@ class _Evaluator:
             b = self.run_copy(b)
         ac, bc, yc = a.c(), b.c(), y.c()
         fn = self.lib.sg_gemm if g.op == "gemm" else self.lib.sg_gemm_batched
-        self.launch(fn(self.ctx.handle, int(g.attrs["ta"]), int(g.attrs["tb"]), C.byref(ac), C.byref(bc), C.byref(yc), ep))
+        self.call(fn, int(g.attrs["ta"]), int(g.attrs["tb"]), C.byref(ac), C.byref(bc), C.byref(yc), ep)
         return y
 
     def _ev_gemm(self, v):
@@ -1053,14 +1085,14 @@ class _Evaluator:
         y = self.out(v.extents, FLOAT)
         xc, yc = xt.c(), y.c()
         ac = addend.c() if addend is not None else None
-        self.launch(self.lib.sg_softmax_lastaxis(self.ctx.handle, C.byref(xc), C.byref(ac) if ac is not None else None, C.byref(yc)))
+        self.call(self.lib.sg_softmax_lastaxis, C.byref(xc), C.byref(ac) if ac is not None else None, C.byref(yc))
         return y
 
     def _ev_softmax_ce(self, v):
         x, lab = self.get(v.inputs[0]), self.get(v.inputs[1])
         y = self.out(v.extents, FLOAT)
         xc, lc, yc = x.c(), lab.c(), y.c()
-        self.launch(self.lib.sg_softmax_cross_entropy(self.ctx.handle, C.byref(xc), C.byref(lc), C.byref(yc)))
+        self.call(self.lib.sg_softmax_cross_entropy, C.byref(xc), C.byref(lc), C.byref(yc))
         return y
 
     def _ev_layer_norm(self, v):
@@ -1069,5 +1101,5 @@ class _Evaluator:
             x = self.run_copy(x)
         y = self.out(v.extents, FLOAT)
         xc, gc, bc, yc = x.c(), g.c(), b.c(), y.c()
-        self.launch(self.lib.sg_layer_norm_lastaxis(self.ctx.handle, C.byref(xc), C.byref(gc), C.byref(bc), C.c_float(v.attrs["eps"]), C.byref(yc)))
+        self.call(self.lib.sg_layer_norm_lastaxis, C.byref(xc), C.byref(gc), C.byref(bc), C.c_float(v.attrs["eps"]), C.byref(yc))
         return y

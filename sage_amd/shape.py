@@ -53,18 +53,25 @@ def norm_axes(axes, bound):
 
 
 def infer_extents(extents, size):
-    """Extent::to_arr with one inferred (-1) entry (shape.rs:540-600)."""
+    """Extent::to_arr (shape.rs:540-640): `size` 0 means "not specified"; one entry may be -1 and is
+    then inferred from `size`; any other non-positive entry is invalid; a specified size must match."""
     extents = [int(e) for e in extents]
-    if extents.count(-1) > 1:
-        raise ShapeError("invalid extents")
-    if -1 in extents:
-        known = 1
-        for e in extents:
-            if e != -1:
-                known *= e
-        if known == 0 or size % known:
-            raise ShapeError("invalid extents")
+    for e in extents:
+        if e < 1 and e != -1:
+            raise ShapeError(f"invalid extent {e}")
+    n_infer = extents.count(-1)
+    if n_infer > 1:
+        raise ShapeError("invalid inference")
+    known = 1
+    for e in extents:
+        if e != -1:
+            known *= e
+    if n_infer == 1:
+        if size == 0 or size % known:
+            raise ShapeError("invalid inference")
         extents[extents.index(-1)] = size // known
+    elif size != 0 and known != size:
+        raise ShapeError(f"size mismatch ({size}, {known})")
     return extents
 
 

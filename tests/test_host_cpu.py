@@ -1,0 +1,225 @@
+"""CPU-only checks: the stride algebra, the C-ABI library (loads, exports every declared symbol),
+the run-time kernel generator (source + gfx950 compile, no GPU needed) and the rule that the
+product never reaches into the oracle."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from sage_amd import abi
+from sage_amd.shape import Shape, ShapeError, default_strides, infer_extents, norm_axes, norm_axis, union
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ------------------------------------------------------------------ shape.rs:707-870
+def test_axis():
+    assert norm_axis(-3, 3) == 0 and norm_axis(-2, 3) == 1 and norm_axis(0, 3) == 0 and norm_axis(1, 3) == 1
+    for a, b in ((0, 0), (-4, 3), (4, 4)):
+        with pytest.raises(ShapeError):
+            norm_axis(a, b)
+    assert norm_axes([-3, -2, -1, 0, 1, 2], 3) == [0, 1, 2, 0, 1, 2]
+    with pytest.raises(ShapeError):
+        norm_axes([-4, -2, -1, 0, 1, 2], 3)
+
+
+def test_extents():
+    assert infer_extents([2, 3, 4], 0) == [2, 3, 4]
+    assert infer_extents([2, 3, 4], 24) == [2, 3, 4]
+    assert infer_extents([-1, 3, 4], 24) == [2, 3, 4]
+    assert infer_extents([2, -1, 4], 24) == [2, 3, 4]
+    assert infer_extents([2, 3, -1], 24) == [2, 3, 4]
+    for ext, size in (([1, 3, -4], 24), ([1, 0, 4], 24), ([1, 3, 4], 24), ([1, 3, 4], 23), ([1, 3, 4], 25),
+                      ([-1, -1, 4], 24), ([-1, 3, 4], 0), ([-1, 3, 4], 25)):
+        with pytest.raises(ShapeError):
+            infer_extents(ext, size)
+
+
+def test_union():
+    assert union([1, 3, 4], [1, 3, 4]) == [1, 3, 4]
+    assert union([5, 6, 1, 3, 4], [1, 3, 4]) == [5, 6, 1, 3, 4]
+    assert union([5, 6, 1, 3, 4], [7, 3, 4]) == [5, 6, 7, 3, 4]
+    assert union([1, 2, 1, 2, 1, 2], [2, 1, 2, 1, 2, 1]) == [2, 2, 2, 2, 2, 2]
+    with pytest.raises(ShapeError):
+        union([2, 3], [4, 3])
+
+
+def test_shape_algebra_against_numpy():
+    """Every layout method against numpy's own stride arithmetic on a real array."""
+    a = np.arange(2 * 3 * 4 * 5, dtype=np.float32).reshape(2, 3, 4, 5)
+    flat = a.reshape(-1)
+
+    def realise(sh):
+        return np.array(np.lib.stride_tricks.as_strided(flat[sh.offset:], sh.extents, [s * 4 for s in sh.strides]))
+
+    s = Shape(a.shape)
+    assert s.strides == [60, 20, 5, 1] == default_strides(a.shape) and s.has_default_strides()
+    assert np.array_equal(realise(s.permute([2, 0, 3, 1])), a.transpose(2, 0, 3, 1))
+    assert np.array_equal(realise(s.swap(1, 3)), a.swapaxes(1, 3))
+    assert np.array_equal(realise(s.select_range(1, 2, 2)), a[:, :, 1:3])
+    assert np.array_equal(realise(s.select(2, 1)), a[:, 2])
+    assert np.array_equal(realise(s.select_range(0, 0, 1).remove(1).insert(0)), a[None, :, 0])
+    e = Shape([3, 1, 5]).expand([2, 1, 3, 9, 5])  # the example in shape.rs:248-249
+    assert e.extents == [2, 1, 3, 9, 5] and e.strides == [0, 0, 5, 0, 1]
+    with pytest.raises(ShapeError):
+        Shape([3, 2]).expand([3, 4])
+    # has_default_strides ignores the offset (shape.rs:134-143); insert() gives stride 0 (shape.rs:190-195)
+    assert s.select_range(1, 1, 0).has_default_strides()
+    assert not Shape([4]).insert(1).has_default_strides()
+    for i in range(s.size()):
+        t = s.permute([3, 1, 0, 2])
+        assert flat[t.translate_default(i)] == a.transpose(3, 1, 0, 2).reshape(-1)[i]
+    inner, outer = s.extract([1, 3], True)
+    assert inner.extents == [3, 5] and inner.strides == [20, 1] and outer.extents == [2, 4] and outer.strides == [60, 5]
+    assert Shape([2, 3]).is_contiguous() and not Shape([2, 3], [6, 1]).is_contiguous()
+    assert not Shape([2, 3]).expand([4, 2, 3]).is_bijective()
+
+
+# ------------------------------------------------------------------ the C-ABI library
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sage_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_symbols()
+    assert len(names) >= 35
+    lib = abi.lib()  # raises if the library is missing or a prototype has no symbol
+    out = subprocess.check_output(["nm", "-D", "--defined-only", abi.LIB_PATH], text=True)
+    exported = set(re.findall(r" T (sg_[a-z0-9_]+)", out))
+    assert set(names) <= exported, sorted(set(names) - exported)
+    assert set(names) == set(abi.PROTOTYPES), (sorted(set(names) ^ set(abi.PROTOTYPES)))
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
+def test_struct_layout_matches_header():
+    assert C.sizeof(abi.sg_tensor) == 8 + 4 + 4 + 8 * 8 + 8 * 8 + 8
+    assert C.sizeof(abi.sg_expr) == 16
+    assert abi.sg_tensor.offset.offset == 144 and abi.sg_tensor.strides.offset == 80
+
+
+def test_no_context_without_gpu_is_an_error_not_a_fallback():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    h = C.c_void_p()
+    assert abi.lib().sg_ctx_create(0, 0, C.byref(h)) == abi.ERR_DEVICE and not h.value
+
+
+def test_product_does_not_touch_the_oracle():
+    for d, _, files in os.walk(os.path.join(ROOT, "sage_amd")):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(d, f)).read()
+                assert "oracle" not in text.replace("CPU oracle", ""), f
+
+
+# ------------------------------------------------------------------ run-time kernel generator
+def desc(extents, strides=None, offset=0, dtype=abi.FLOAT):
+    t = abi.sg_tensor()
+    t.base = None
+    t.dtype = dtype
+    t.rank = len(extents)
+    st = default_strides(extents) if strides is None else strides
+    for i, (e, s) in enumerate(zip(extents, st)):
+        t.extents[i], t.strides[i] = e, s
+    t.offset = offset
+    return t
+
+
+def prog(*items):
+    arr = (abi.sg_expr * len(items))()
+    for i, (k, o, d, b) in enumerate(items):
+        arr[i].kind, arr[i].op, arr[i].dtype, arr[i].bits = k, o, d, b
+    return arr, len(items)
+
+
+def source(items, ins, out):
+    arr, n = prog(*items)
+    buf = C.create_string_buffer(1 << 16)
+    dt = C.c_int32(-1)
+    inarr = (abi.sg_tensor * max(1, len(ins)))(*ins)
+    rc = abi.lib().sg_map_source(None, arr, n, inarr, len(ins), C.byref(out), buf, len(buf), C.byref(dt))
+    return rc, buf.value.decode(), dt.value
+
+
+def compiles(src):
+    log = C.create_string_buffer(1 << 14)
+    rc = abi.lib().sg_map_compile_only(src.encode(), log, len(log))
+    assert rc == abi.OK, log.value.decode()
+
+
+INP = lambda i: (abi.EXPR_INPUT, i, 0, 0)
+UN = lambda n: (abi.EXPR_UNARY, abi.U[n], 0, 0)
+BIN = lambda n: (abi.EXPR_BINARY, abi.B[n], 0, 0)
+LITF = lambda v: (abi.EXPR_LITERAL, 0, abi.FLOAT, int(np.float32(v).view(np.uint32)))
+COND = (abi.EXPR_TERNARY, 0, 0, 0)
+
+
+def test_map_source_vector_path_and_compile():
+    """exp(x0 - x1), x1 broadcast per row: 16-byte loads for x0, one scalar load for x1."""
+    x0 = desc([8192, 1024])
+    x1 = desc([8192, 1024], [1, 0])
+    rc, src, dt = source([UN("exp"), BIN("sub"), INP(0), INP(1)], [x0, x1], desc([8192, 1024]))
+    assert rc == abi.OK and dt == abi.FLOAT
+    assert "const float4 v0" in src and "const float s1" in src and "expf((x0 - x1))" in src
+    compiles(src)
+
+
+def test_map_source_scalar_path_for_transposed_operand():
+    xt = desc([6, 4], [1, 6])
+    rc, src, _ = source([UN("sin"), INP(0)], [xt], desc([6, 4]))
+    assert rc == abi.OK and "float4" not in src.split("extern")[1] and "sinf(x0)" in src
+    compiles(src)
+
+
+def test_map_source_collapses_dense_axes():
+    rc, src, _ = source([BIN("add"), INP(0), INP(1)], [desc([4, 8, 16, 32]), desc([4, 8, 16, 32])], desc([4, 8, 16, 32]))
+    assert rc == abi.OK and "#define ND 1" in src
+    bias = desc([32, 128, 768], [0, 0, 1])
+    rc, src, _ = source([BIN("add"), INP(0), INP(1)], [desc([32, 128, 768]), bias], desc([32, 128, 768]))
+    assert rc == abi.OK and "#define ND 2" in src and "const float4 v1" in src
+
+
+def test_every_map_operator_compiles_for_gfx950():
+    """One kernel holding all 27 unary operators and one holding the binary ones + cond."""
+    items = []
+    for name in abi.UNARY:
+        if name in ("not",):
+            continue
+        items = [UN(name)] + (items or [INP(0)])
+    items = [UN("cast_float"), UN("not")] + items
+    rc, src, dt = source(items, [desc([64, 64])], desc([64, 64]))
+    assert rc == abi.OK and dt == abi.FLOAT, src
+    compiles(src)
+    e = [INP(0)]
+    for name in ("add", "sub", "div", "mul", "pow", "min", "max"):
+        e = [BIN(name)] + e + [INP(1)]
+    cmp_ = lambda n: [BIN(n), INP(0), INP(1)]
+    c = [BIN("and")] + cmp_("gt") + [BIN("or")] + cmp_("le") + [BIN("ne")] + cmp_("eq") + cmp_("ge")
+    rc, src, dt = source([COND] + c + e + [LITF(1.5)], [desc([10, 7]), desc([10, 7])], desc([10, 7]))
+    assert rc == abi.OK and dt == abi.FLOAT, src
+    compiles(src)
+
+
+def test_map_dtype_rules_and_errors():
+    """map.rs:464-470, 491-501, 869-870; mod has no kernel (map.rs:275)."""
+    f, i, u = desc([4, 4]), desc([4, 4], dtype=abi.INT), desc([4, 4], dtype=abi.UINT)
+    assert source([BIN("gt"), INP(0), INP(1)], [f, f], u)[2] == abi.UINT
+    assert source([UN("cast_int"), INP(0)], [f], i)[2] == abi.INT
+    assert source([UN("abs"), INP(0)], [i], i)[2] == abi.INT
+    assert source([UN("exp"), INP(0)], [i], f)[2] == abi.FLOAT
+    assert source([UN("not"), INP(0)], [f], u)[2] == abi.UINT
+    assert source([BIN("add"), INP(0), INP(1)], [f, i], f)[0] == abi.ERR_DTYPE
+    assert source([COND, INP(0), INP(1), INP(1)], [f, f], f)[0] == abi.ERR_DTYPE
+    assert source([BIN("gt"), INP(0), INP(1)], [f, f], f)[0] == abi.ERR_DTYPE  # output must be uint
+    assert source([BIN("mod"), INP(0), INP(1)], [f, f], f)[0] == abi.ERR_ARG
+    assert source([BIN("add"), INP(0)], [f], f)[0] == abi.ERR_ARG                # program ends early
+    assert source([UN("exp"), INP(0)], [desc([4, 5])], f)[0] == abi.ERR_SHAPE    # ops.rs:174
+    assert source([UN("exp"), INP(0)], [f], desc([4, 4], [1, 4]))[0] == abi.ERR_SHAPE  # output not dense
+    assert source([UN("exp"), INP(0)], [desc([4, 4], dtype=abi.LONG)], f)[0] == abi.ERR_DTYPE

@@ -9,12 +9,18 @@
 // Design:
 //   * One workgroup = 4 wavefronts computes a BM x BN tile of C; a wavefront owns a
 //     (BM/WAVES_M) x (BN/WAVES_N) sub-tile as TM x TN accumulators of 32x32 (16 VGPRs each).
-//   * K is walked in slabs of 32.  A slab of A and of B is fetched from global memory with
-//     16-byte loads into registers while the previous slab is being multiplied, then written to
-//     LDS as As[k][m], Bs[k][n] — the layout in which one MFMA operand fetch is a conflict-free
-//     ds_read of 32 consecutive floats per half-wave.  Operands that are contiguous along k
-//     (row-major A, transposed B) are transposed on their way into LDS, so all four transpose
-//     modes, and arbitrarily strided batches, run the same inner loop without any pre-copy.
+//   * K is walked in slabs of 16 through a double-buffered LDS: while slab kt is multiplied out of
+//     one buffer, slab kt+1 (fetched one iteration earlier into registers) is written to the other
+//     and slab kt+2 is being fetched from global memory; one barrier per slab.
+//   * Global loads and LDS stores are 16 bytes wide for every layout.  An operand that is
+//     contiguous along k (row-major A, transposed B) is kept in LDS as [row][k] and one MFMA operand
+//     fetch is a 16-byte read of 4 consecutive k; an operand contiguous along its rows is kept as
+//     [k][row] and fetched 4 bytes at a time.  Both orders are bank-conflict free, so all four
+//     transpose modes and arbitrarily strided batches run the same loop without any pre-copy or
+//     transposition.  (The k index a lane multiplies at step s of a group of four steps is
+//     8g + 4*(lane/32) + s for both operands, which is all the MFMA needs.)
+//   * Tiles that lie fully inside aligned matrices run an instantiation with no bounds checks at
+//     all; only edge shapes pay for guarded, zero-filling loads.
 //   * Workgroup ids are remapped so that the ids one XCD receives (id mod 8) cover a compact block
 //     of tiles, which keeps the A/B panels a tile group shares inside that XCD's L2.
 //   * The epilogue applies alpha, bias[n], activation and a residual while the accumulators are
@@ -26,9 +32,11 @@
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));  // native vector: stays in registers
 
-constexpr int BK = 32;
-constexpr int PAD = 4;
+constexpr int BK = 16;   // k-slab
+constexpr int KPAD = 4;  // row padding of [row][k] LDS tiles (floats)
+constexpr int RPAD = 4;  // row padding of [k][row] LDS tiles (floats)
 constexpr int NTHREADS = 256;
 constexpr int NUM_XCD = 8;
 
@@ -52,44 +60,79 @@ __device__ __forceinline__ float apply_act(float v, int act) {
     return v;
 }
 
-// Fetch a ROWS x BK slab (rows = m or n indices) into registers, then store it to LDS as [k][row].
-template <int ROWS, bool K_CONTIG> struct Slab {
-    static constexpr int NV = ROWS * BK / 4 / NTHREADS;  // float4 per thread
-    static constexpr int LD = ROWS + PAD;
-    float4 r[NV];
+// One operand tile (ROWS x BK; rows are m or n indices) on its way from global memory to LDS.
+// K_CONTIG: the operand is contiguous along k in global memory.  The tile is then kept in LDS as
+// [row][k] (row stride BK+KPAD floats) and an MFMA operand fetch is ONE 16-byte read of 4
+// consecutive k; with the padding, 8 consecutive rows cover all 32 banks.  Otherwise the operand is
+// contiguous along its rows, the tile is kept as [k][row] (row stride ROWS+RPAD) and a fetch is a
+// 4-byte read of 32 consecutive floats per half-wave.  Either way global loads and LDS stores are
+// 16 bytes wide and no transposition happens on the way.
+template <int ROWS, bool K_CONTIG> struct Tile {
+    static constexpr int TOTAL = ROWS * BK / 4;                      // float4 per slab
+    static constexpr int NV = (TOTAL + NTHREADS - 1) / NTHREADS;     // float4 per thread (last may be partial)
+    static constexpr int LD = K_CONTIG ? BK + KPAD : ROWS + RPAD;
+    static constexpr int SIZE = K_CONTIG ? ROWS * LD : BK * LD;      // floats
 
-    __device__ __forceinline__ void load(const float *base, int row0, int k0, int row_lim, int k_lim, int64_t s_row, int64_t s_k,
-                                         int vec_ok, int tid) {
+    // element (row, k) of the slab handled by slot f of this thread
+    __device__ static __forceinline__ void where(int f, int &row, int &k) {
+        if (K_CONTIG) {
+            row = f / (BK / 4);
+            k = (f % (BK / 4)) * 4;
+        } else {
+            k = f / (ROWS / 4);
+            row = (f % (ROWS / 4)) * 4;
+        }
+    }
+    __device__ static __forceinline__ int lds_at(int row, int k) { return K_CONTIG ? row * LD + k : k * LD + row; }
+
+    // unguarded: whole tile inside the matrix, 16-byte aligned
+    __device__ static __forceinline__ void load_fast(f32x4 (&r)[NV], const float *base, int row0, int k0, int64_t s_row, int64_t s_k, int tid) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int f = tid + i * NTHREADS;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (K_CONTIG) {
-                const int kq = f % (BK / 4), row = f / (BK / 4);
-                const int gr = row0 + row, gk = k0 + kq * 4;
-                if (gr < row_lim) {
-                    const float *p = base + (int64_t)gr * s_row + gk;
-                    if (vec_ok && gk + 3 < k_lim) {
-                        v = *reinterpret_cast<const float4 *>(p);
-                    } else {
-                        if (gk + 0 < k_lim) v.x = p[0];
-                        if (gk + 1 < k_lim) v.y = p[1];
-                        if (gk + 2 < k_lim) v.z = p[2];
-                        if (gk + 3 < k_lim) v.w = p[3];
+            if (TOTAL % NTHREADS == 0 || f < TOTAL) {
+                int row, k;
+                where(f, row, k);
+                const float *p = K_CONTIG ? base + (int64_t)(row0 + row) * s_row + (k0 + k) : base + (int64_t)(k0 + k) * s_k + (row0 + row);
+                r[i] = *reinterpret_cast<const f32x4 *>(p);
+            }
+        }
+    }
+
+    // guarded: zero-fill outside [row_lim) x [k_lim), scalar loads when 16-byte loads are not legal
+    __device__ static __forceinline__ void load_guarded(f32x4 (&r)[NV], const float *base, int row0, int k0, int row_lim, int k_lim, int64_t s_row,
+                                                        int64_t s_k, int vec_ok, int tid) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int f = tid + i * NTHREADS;
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (TOTAL % NTHREADS == 0 || f < TOTAL) {
+                int row, k;
+                where(f, row, k);
+                const int gr = row0 + row, gk = k0 + k;
+                if (K_CONTIG) {
+                    if (gr < row_lim) {
+                        const float *p = base + (int64_t)gr * s_row + gk;
+                        if (vec_ok && gk + 3 < k_lim) {
+                            v = *reinterpret_cast<const f32x4 *>(p);
+                        } else {
+                            if (gk + 0 < k_lim) v.x = p[0];
+                            if (gk + 1 < k_lim) v.y = p[1];
+                            if (gk + 2 < k_lim) v.z = p[2];
+                            if (gk + 3 < k_lim) v.w = p[3];
+                        }
                     }
-                }
-            } else {
-                const int rq = f % (ROWS / 4), k = f / (ROWS / 4);
-                const int gr = row0 + rq * 4, gk = k0 + k;
-                if (gk < k_lim) {
-                    const float *p = base + (int64_t)gk * s_k + gr;
-                    if (vec_ok && gr + 3 < row_lim) {
-                        v = *reinterpret_cast<const float4 *>(p);
-                    } else {
-                        if (gr + 0 < row_lim) v.x = p[0];
-                        if (gr + 1 < row_lim) v.y = p[1];
-                        if (gr + 2 < row_lim) v.z = p[2];
-                        if (gr + 3 < row_lim) v.w = p[3];
+                } else {
+                    if (gk < k_lim) {
+                        const float *p = base + (int64_t)gk * s_k + gr;
+                        if (vec_ok && gr + 3 < row_lim) {
+                            v = *reinterpret_cast<const f32x4 *>(p);
+                        } else {
+                            if (gr + 0 < row_lim) v.x = p[0];
+                            if (gr + 1 < row_lim) v.y = p[1];
+                            if (gr + 2 < row_lim) v.z = p[2];
+                            if (gr + 3 < row_lim) v.w = p[3];
+                        }
                     }
                 }
             }
@@ -97,33 +140,41 @@ template <int ROWS, bool K_CONTIG> struct Slab {
         }
     }
 
-    __device__ __forceinline__ void store(float *lds, int tid) const {
+    __device__ static __forceinline__ void store(const f32x4 (&r)[NV], float *lds, int tid) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int f = tid + i * NTHREADS;
-            if (K_CONTIG) {
-                const int kq = f % (BK / 4), row = f / (BK / 4);
-                lds[(kq * 4 + 0) * LD + row] = r[i].x;
-                lds[(kq * 4 + 1) * LD + row] = r[i].y;
-                lds[(kq * 4 + 2) * LD + row] = r[i].z;
-                lds[(kq * 4 + 3) * LD + row] = r[i].w;
-            } else {
-                const int rq = f % (ROWS / 4), k = f / (ROWS / 4);
-                *reinterpret_cast<float4 *>(&lds[k * LD + rq * 4]) = r[i];
+            if (TOTAL % NTHREADS == 0 || f < TOTAL) {
+                int row, k;
+                where(f, row, k);
+                *reinterpret_cast<f32x4 *>(&lds[lds_at(row, k)]) = r[i];
             }
+        }
+    }
+
+    // MFMA operands of one group of 4 k-steps for the 32 rows starting at `col0`: step s of group g
+    // multiplies k = 8g + 4*(lane/32) + s.
+    __device__ static __forceinline__ void fetch(const float *lds, int col, int g, int khalf, float out[4]) {
+        if (K_CONTIG) {
+            const f32x4 v = *reinterpret_cast<const f32x4 *>(&lds[col * LD + 8 * g + 4 * khalf]);
+            out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) out[s] = lds[(8 * g + 4 * khalf + s) * LD + col];
         }
     }
 };
 
-template <int BM, int BN, int WAVES_M, bool A_KC, bool B_NC>
+template <int BM, int BN, int WAVES_M, bool A_KC, bool B_NC, bool GUARD>
 __global__ void __launch_bounds__(NTHREADS) gemm_mfma_kernel(const GemmP p) {
     constexpr int WAVES_N = 4 / WAVES_M;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
-    constexpr int LDA = BM + PAD, LDB = BN + PAD;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA block");
-    __shared__ __attribute__((aligned(16))) float As[BK * LDA];
-    __shared__ __attribute__((aligned(16))) float Bs[BK * LDB];
+    typedef Tile<BM, A_KC> TA;
+    typedef Tile<BN, !B_NC> TB;
+    __shared__ __attribute__((aligned(16))) float lds_a[2][TA::SIZE];
+    __shared__ __attribute__((aligned(16))) float lds_b[2][TB::SIZE];
 
     // ---- which tile: spread consecutive ids over XCDs, then walk tiles in groups of 8 tile-rows
     const int ntiles = p.tiles_m * p.tiles_n;
@@ -159,35 +210,54 @@ __global__ void __launch_bounds__(NTHREADS) gemm_mfma_kernel(const GemmP p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    Slab<BM, A_KC> sa;
-    Slab<BN, !B_NC> sb;
-    sa.load(A, m0, 0, p.M, p.K, p.a_sm, p.a_sk, p.vec_a, tid);
-    sb.load(B, n0, 0, p.N, p.K, p.b_sn, p.b_sk, p.vec_b, tid);
+    f32x4 ra[TA::NV], rb[TB::NV];
+#define SG_LOAD_SLAB(k0)                                                                       \
+    do {                                                                                       \
+        if (GUARD) {                                                                           \
+            TA::load_guarded(ra, A, m0, (k0), p.M, p.K, p.a_sm, p.a_sk, p.vec_a, tid);              \
+            TB::load_guarded(rb, B, n0, (k0), p.N, p.K, p.b_sn, p.b_sk, p.vec_b, tid);              \
+        } else {                                                                               \
+            TA::load_fast(ra, A, m0, (k0), p.a_sm, p.a_sk, tid);                                    \
+            TB::load_fast(rb, B, n0, (k0), p.b_sn, p.b_sk, tid);                                    \
+        }                                                                                      \
+    } while (0)
+
+    // LDS is double-buffered: slab kt is multiplied out of buffer kt&1 while slab kt+1 (already in
+    // registers) is written to the other buffer and slab kt+2 is fetched from global memory.
+    const int nk = (p.K + BK - 1) / BK;
+    SG_LOAD_SLAB(0);
+    TA::store(ra, lds_a[0], tid);
+    TB::store(rb, lds_b[0], tid);
+    if (nk > 1) SG_LOAD_SLAB(BK);
+    __syncthreads();
 
     const int a_col = wm * WM + (lane & 31), b_col = wn * WN + (lane & 31), khalf = lane >> 5;
-    for (int k0 = 0; k0 < p.K; k0 += BK) {
-        __syncthreads();
-        sa.store(As, tid);
-        sb.store(Bs, tid);
-        __syncthreads();
-        if (k0 + BK < p.K) {
-            sa.load(A, m0, k0 + BK, p.M, p.K, p.a_sm, p.a_sk, p.vec_a, tid);
-            sb.load(B, n0, k0 + BK, p.N, p.K, p.b_sn, p.b_sk, p.vec_b, tid);
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) {
+            TA::store(ra, lds_a[cur ^ 1], tid);
+            TB::store(rb, lds_b[cur ^ 1], tid);
+            if (kt + 2 < nk) SG_LOAD_SLAB((kt + 2) * BK);
         }
+        const float *as = lds_a[cur], *bs = lds_b[cur];
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-            float a[TM], b[TN];
+        for (int g = 0; g < BK / 8; ++g) {
+            float a[TM][4], b[TN][4];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) a[i] = As[(kk + khalf) * LDA + a_col + i * 32];
+            for (int i = 0; i < TM; ++i) TA::fetch(as, a_col + i * 32, g, khalf, a[i]);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) b[j] = Bs[(kk + khalf) * LDB + b_col + j * 32];
+            for (int j = 0; j < TN; ++j) TB::fetch(bs, b_col + j * 32, g, khalf, b[j]);
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+            for (int s = 0; s < 4; ++s)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
         }
+        __syncthreads();
     }
 
+#undef SG_LOAD_SLAB
     // ---- epilogue: element r of a 32x32 block sits at row (r/4)*8 + (lane/32)*4 + r%4, col lane%32
     float *C = p.C + b0 * p.c_sb0 + b1 * p.c_sb1;
     const float *R = p.res ? p.res + b0 * p.r_sb0 + b1 * p.r_sb1 : nullptr;
@@ -215,21 +285,31 @@ __global__ void __launch_bounds__(NTHREADS) gemm_mfma_kernel(const GemmP p) {
     }
 }
 
+template <int BM, int BN, int WAVES_M, bool GUARD>
+void launch_layouts(sg_ctx *ctx, const GemmP &p, dim3 grid, bool a_kc, bool b_nc) {
+    dim3 block(NTHREADS);
+    if (a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD>), grid, block, 0, ctx->stream, p);
+    else if (a_kc && !b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, false, GUARD>), grid, block, 0, ctx->stream, p);
+    else if (!a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, true, GUARD>), grid, block, 0, ctx->stream, p);
+    else hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, false, GUARD>), grid, block, 0, ctx->stream, p);
+}
+
+// GUARD = false needs every tile to lie fully inside the matrices and 16-byte loads to be legal.
+bool needs_guard(const GemmP &p, int bm, int bn) {
+    return p.M % bm != 0 || p.N % bn != 0 || p.K % BK != 0 || !p.vec_a || !p.vec_b;
+}
+
 template <int BM, int BN, int WAVES_M>
 int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
-    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch), block(NTHREADS);
-    if (a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true>), grid, block, 0, ctx->stream, p);
-    else if (a_kc && !b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, false>), grid, block, 0, ctx->stream, p);
-    else if (!a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, true>), grid, block, 0, ctx->stream, p);
-    else hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, false>), grid, block, 0, ctx->stream, p);
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
+    if (needs_guard(p, BM, BN)) launch_layouts<BM, BN, WAVES_M, true>(ctx, p, grid, a_kc, b_nc);
+    else launch_layouts<BM, BN, WAVES_M, false>(ctx, p, grid, a_kc, b_nc);
     SG_CHECK_LAUNCH(ctx, "gemm");
     return SG_OK;
 }
 
-// Tile choice: the largest tile that still gives every CU at least one workgroup, preferring an
-// exact multiple of the CU count (no partially filled last round of workgroups).
 struct TileCfg { int bm, bn, waves_m; };
 const TileCfg kTileCfgs[] = {{128, 128, 2}, {128, 96, 4}, {128, 64, 2}, {64, 64, 2}};
 
@@ -351,10 +431,11 @@ int check_f32(sg_ctx *ctx, const sg_tensor *a, const sg_tensor *b, const sg_tens
 extern "C" int sg_gemm_kernel_name(sg_ctx *ctx, int64_t M, int64_t N, int64_t K, int64_t batch, int a_k_contiguous,
                                    int b_n_contiguous, char *buf, uint64_t cap) {
     if (!ctx || !buf || cap < 8) return SG_ERR_ARG;
-    (void)K;
     const TileCfg &t = kTileCfgs[choose_tile(ctx->num_cus, (int)M, (int)N, (int)batch)];
-    snprintf(buf, cap, "gemm_mfma_kernel<%d, %d, %d, %s, %s>", t.bm, t.bn, t.waves_m, a_k_contiguous ? "true" : "false",
-             b_n_contiguous ? "true" : "false");
+    // the fast instantiation when the shape tiles exactly (operands assumed 16-byte aligned here)
+    const bool guard = M % t.bm != 0 || N % t.bn != 0 || K % BK != 0;
+    snprintf(buf, cap, "gemm_mfma_kernel<%d, %d, %d, %s, %s, %s>", t.bm, t.bn, t.waves_m, a_k_contiguous ? "true" : "false",
+             b_n_contiguous ? "true" : "false", guard ? "true" : "false");
     return SG_OK;
 }
 

@@ -144,6 +144,7 @@ template <class A, class B> __device__ __forceinline__ auto sg_max(A a, B b) -> 
 struct MapPlan {
     int ndim = 1;
     int vec = 1;
+    int unroll = 1;  // independent vectors per thread (more bytes in flight for large maps)
     uint32_t ext[SG_MAX_RANK];
     uint32_t stride[SG_MAX_MAP_INPUTS][SG_MAX_RANK];
     bool direct[SG_MAX_MAP_INPUTS];
@@ -202,6 +203,10 @@ void plan_map(const sg_tensor *in, int n_in, const sg_tensor *out, MapPlan &pl) 
         }
     }
     pl.vec = vec_ok ? 4 : 1;
+    int64_t total = 1;
+    for (int a = 0; a < nd; ++a) total *= ext[a];
+    total /= pl.vec;
+    pl.unroll = total >= (1 << 20) ? 4 : total >= (1 << 18) ? 2 : 1;
     for (int a = 0; a < nd; ++a) {
         pl.ext[a] = (uint32_t)ext[a];
         for (int k = 0; k < n_in; ++k) pl.stride[k][a] = (uint32_t)st[k][a];
@@ -221,7 +226,8 @@ std::string gen_source(const std::string &expr, const sg_tensor *in, int n_in, i
     s << "extern \"C\" __global__ void __launch_bounds__(256) sg_map(";
     for (int k = 0; k < n_in; ++k) s << "const " << ctype(in[k].dtype) << " *__restrict__ b" << k << ", ";
     s << ctype(out_dt) << " *__restrict__ yb, const MapParams p) {\n";
-    s << "  uint gid = blockIdx.x * 256u + threadIdx.x;\n  if (gid >= p.total) return;\n";
+    s << "  const uint base = blockIdx.x * " << 256 * pl.unroll << "u + threadIdx.x;\n";
+    s << "#pragma unroll\n  for (uint u = 0; u < " << pl.unroll << "u; ++u) {\n  const uint gid = base + u * 256u;\n  if (gid < p.total) {\n";
     if (pl.need_coords) {
         // coordinates in units of V elements along the innermost axis
         s << "  uint rem = gid, q;\n";
@@ -269,7 +275,7 @@ std::string gen_source(const std::string &expr, const sg_tensor *in, int n_in, i
         }
         s << "  *reinterpret_cast<" << odt << "4 *>(yb + p.yoff + gid * 4u) = r;\n";
     }
-    s << "}\n";
+    s << "  }\n  }\n}\n";
     return s.str();
 }
 
@@ -423,7 +429,8 @@ extern "C" int sg_map(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_ten
     ptrs[n_in] = out->base;
     args.push_back(&ptrs[n_in]);
     args.push_back(params.data());
-    const unsigned grid = (unsigned)((total + 255) / 256);
+    const int64_t per_block = 256 * pl.unroll;
+    const unsigned grid = (unsigned)((total + per_block - 1) / per_block);
     SG_HIP(ctx, hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr));
     return SG_OK;
 }

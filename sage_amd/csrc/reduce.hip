@@ -187,21 +187,31 @@ __global__ void __launch_bounds__(256) reduce_arg_row_kernel(const T *__restrict
     if (lane == 0) y[row] = arg;
 }
 
-// ---- fused row operators: each wavefront keeps one row in registers ---------------------------
-// Row elements are dealt to lanes as 16-byte chunks: chunk j of lane l covers columns
-// (j*64 + l)*4 .. +3, so every load instruction of the wavefront covers 1 KiB of consecutive bytes.
+// ---- fused row operators: rows stay in registers between the read and the write ---------------
+// A row is dealt to LPR lanes (a power of two, 4..64) as 16-byte chunks: chunk j of lane l covers
+// columns (j*LPR + l)*4 .. +3.  Long rows use the whole wavefront (LPR = 64) and several chunks per
+// lane; short rows use a fraction of it, so one wavefront carries 64/LPR rows and every load
+// instruction still moves 1 KiB.  Reductions run over the LPR lanes of a row with xor shuffles.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 template <int NCHUNK> struct RowRegs {
-    float4 v[NCHUNK];
+    f32x4 v[NCHUNK];
 };
 
-template <int NCHUNK>
-__device__ __forceinline__ void load_row(const float *p, uint32_t len, int lane, RowRegs<NCHUNK> &r, float fill) {
+template <int NCHUNK, int LPR>
+__device__ __forceinline__ void load_row(const float *p, uint32_t len, int li, RowRegs<NCHUNK> &r, float fill) {
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
-        uint32_t c = (j * WAVE + lane) * 4u;
-        if (c < len) r.v[j] = *reinterpret_cast<const float4 *>(p + c);
-        else r.v[j] = make_float4(fill, fill, fill, fill);
+        uint32_t c = (j * LPR + li) * 4u;
+        if (c < len) r.v[j] = *reinterpret_cast<const f32x4 *>(p + c);
+        else r.v[j] = f32x4{fill, fill, fill, fill};
     }
+}
+
+template <int OP, int LPR> __device__ __forceinline__ float seg_reduce(float v) {
+#pragma unroll
+    for (int m = LPR / 2; m >= 1; m >>= 1) v = combine<OP, float>(v, shfl_xor(v, m));
+    return v;
 }
 
 struct BDims {  // broadcastable operand: strides over the row index space + inner stride
@@ -212,26 +222,27 @@ struct BDims {  // broadcastable operand: strides over the row index space + inn
 
 // softmax(x + addend) over the last axis (nn.rs:42-56).  The shift is max(0, row max), not the row
 // max: the reference's max accumulator starts at literal 0 (reduce.rs:282), and using the same
-// shift keeps even the underflow behaviour of rows far below zero identical.
-template <int NCHUNK, bool HAS_ADD>
+// shift keeps even the underflow behaviour of rows far below zero identical.  The quotient y/sum is
+// formed as y * (1/sum): one division per row instead of one per element.
+template <int NCHUNK, int LPR, bool HAS_ADD>
 __global__ void __launch_bounds__(256) softmax_row_kernel(const float *__restrict__ x, const float *__restrict__ add,
                                                           float *__restrict__ y, uint32_t n_rows, uint32_t len,
                                                           uint32_t x_off, Dims xo, BDims ao, uint32_t y_off) {
-    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
-    const uint32_t row = blockIdx.x * 4u + wave;
+    constexpr int RPW = WAVE / LPR;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, li = lane % LPR;
+    const uint32_t row = (blockIdx.x * 4u + wave) * RPW + lane / LPR;
     if (row >= n_rows) return;
     const float *p = x + x_off + decompose(xo, row);
     RowRegs<NCHUNK> r;
-    load_row<NCHUNK>(p, len, lane, r, -__builtin_inff());
+    load_row<NCHUNK, LPR>(p, len, li, r, -__builtin_inff());
     if (HAS_ADD) {
         const float *a = add + ao.off + decompose(ao.outer, row);
 #pragma unroll
         for (int j = 0; j < NCHUNK; ++j) {
-            uint32_t c = (j * WAVE + lane) * 4u;
+            uint32_t c = (j * LPR + li) * 4u;
             if (c < len) {
                 if (ao.inner_stride == 1) {
-                    float4 t = *reinterpret_cast<const float4 *>(a + c);
-                    r.v[j].x += t.x; r.v[j].y += t.y; r.v[j].z += t.z; r.v[j].w += t.w;
+                    r.v[j] += *reinterpret_cast<const f32x4 *>(a + c);
                 } else {
                     r.v[j].x += a[(c + 0) * ao.inner_stride]; r.v[j].y += a[(c + 1) * ao.inner_stride];
                     r.v[j].z += a[(c + 2) * ao.inner_stride]; r.v[j].w += a[(c + 3) * ao.inner_stride];
@@ -242,7 +253,7 @@ __global__ void __launch_bounds__(256) softmax_row_kernel(const float *__restric
     float m = -__builtin_inff();
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) m = fmaxf(fmaxf(fmaxf(fmaxf(m, r.v[j].x), r.v[j].y), r.v[j].z), r.v[j].w);
-    m = fmaxf(wave_reduce<OP_MAX, float>(m), 0.0f);
+    m = fmaxf(seg_reduce<OP_MAX, LPR>(m), 0.0f);
     float s = 0.0f;
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
@@ -250,15 +261,13 @@ __global__ void __launch_bounds__(256) softmax_row_kernel(const float *__restric
         r.v[j].z = expf(r.v[j].z - m); r.v[j].w = expf(r.v[j].w - m);
         s += (r.v[j].x + r.v[j].y) + (r.v[j].z + r.v[j].w);
     }
-    s = wave_reduce<OP_SUM, float>(s);
+    s = seg_reduce<OP_SUM, LPR>(s);
+    const float inv = 1.0f / s;
     float *q = y + y_off + (size_t)row * len;
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
-        uint32_t c = (j * WAVE + lane) * 4u;
-        if (c < len) {
-            float4 o = make_float4(r.v[j].x / s, r.v[j].y / s, r.v[j].z / s, r.v[j].w / s);
-            *reinterpret_cast<float4 *>(q + c) = o;
-        }
+        uint32_t c = (j * LPR + li) * 4u;
+        if (c < len) *reinterpret_cast<f32x4 *>(q + c) = r.v[j] * inv;
     }
 }
 
@@ -291,28 +300,28 @@ __global__ void __launch_bounds__(256) softmax_row_generic_kernel(const float *_
 
 // softmax_cross_entropy (nn.rs:58-82): c = max(x), lse = log(sum exp(x-c)) + c,
 // loss = -(x[label] - lse).  Same operation order as the composition.
-template <int NCHUNK>
+template <int NCHUNK, int LPR>
 __global__ void __launch_bounds__(256) softmax_ce_row_kernel(const float *__restrict__ x, const uint32_t *__restrict__ labels,
                                                              float *__restrict__ loss, uint32_t n_rows, uint32_t len,
                                                              uint32_t x_off, uint32_t x_row_stride, uint32_t l_off,
                                                              uint32_t l_stride, uint32_t y_off) {
-    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
-    const uint32_t row = blockIdx.x * 4u + wave;
+    constexpr int RPW = WAVE / LPR;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, li = lane % LPR;
+    const uint32_t row = (blockIdx.x * 4u + wave) * RPW + lane / LPR;
     if (row >= n_rows) return;
     const float *p = x + x_off + (size_t)row * x_row_stride;
     RowRegs<NCHUNK> r;
-    load_row<NCHUNK>(p, len, lane, r, -__builtin_inff());
+    load_row<NCHUNK, LPR>(p, len, li, r, -__builtin_inff());
     float m = -__builtin_inff();
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) m = fmaxf(fmaxf(fmaxf(fmaxf(m, r.v[j].x), r.v[j].y), r.v[j].z), r.v[j].w);
-    m = wave_reduce<OP_MAX, float>(m);
-    m = fmaxf(m, 0.0f);  // the reference's max accumulator starts at 0 (reduce.rs:282)
+    m = fmaxf(seg_reduce<OP_MAX, LPR>(m), 0.0f);  // the reference's max accumulator starts at 0 (reduce.rs:282)
     float s = 0.0f;
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j)
         s += (expf(r.v[j].x - m) + expf(r.v[j].y - m)) + (expf(r.v[j].z - m) + expf(r.v[j].w - m));
-    s = wave_reduce<OP_SUM, float>(s);
-    if (lane == 0) {
+    s = seg_reduce<OP_SUM, LPR>(s);
+    if (li == 0) {
         const uint32_t label = labels[l_off + (size_t)row * l_stride];
         const float lse = logf(s) + m;
         loss[y_off + row] = -(p[label] - lse);
@@ -347,48 +356,52 @@ __global__ void __launch_bounds__(256) softmax_ce_row_generic_kernel(const float
 }
 
 // layer_norm over the last axis (nn.rs:84-100): mean = S1/n, var = S2/n - mean^2,
-// y = (x - mean) / sqrt(var + eps) * gamma + beta, with the reference's operation order.
-template <int NCHUNK>
+// y = (x - mean) / sqrt(var + eps) * gamma + beta.  The division by sqrt(var+eps) is applied as a
+// multiplication by its reciprocal (one division per row); everything else keeps the reference's
+// operation order.
+template <int NCHUNK, int LPR>
 __global__ void __launch_bounds__(256) layer_norm_row_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
                                                              const float *__restrict__ beta, float *__restrict__ y,
                                                              uint32_t n_rows, uint32_t len, uint32_t x_off, Dims xo,
                                                              uint32_t g_off, uint32_t g_stride, uint32_t b_off, uint32_t b_stride,
                                                              float eps, uint32_t y_off) {
-    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
-    const uint32_t row = blockIdx.x * 4u + wave;
+    constexpr int RPW = WAVE / LPR;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, li = lane % LPR;
+    const uint32_t row = (blockIdx.x * 4u + wave) * RPW + lane / LPR;
     if (row >= n_rows) return;
     const float *p = x + x_off + decompose(xo, row);
     RowRegs<NCHUNK> r;
-    load_row<NCHUNK>(p, len, lane, r, 0.0f);
+    load_row<NCHUNK, LPR>(p, len, li, r, 0.0f);
     float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
         s1 += (r.v[j].x + r.v[j].y) + (r.v[j].z + r.v[j].w);
         s2 += (r.v[j].x * r.v[j].x + r.v[j].y * r.v[j].y) + (r.v[j].z * r.v[j].z + r.v[j].w * r.v[j].w);
     }
-    s1 = wave_reduce<OP_SUM, float>(s1);
-    s2 = wave_reduce<OP_SUM, float>(s2);
+    s1 = seg_reduce<OP_SUM, LPR>(s1);
+    s2 = seg_reduce<OP_SUM, LPR>(s2);
     const float n = (float)len;
     const float mean = s1 / n;
     const float var = s2 / n - mean * mean;
-    const float denom = sqrtf(var + eps);
+    const float inv = 1.0f / sqrtf(var + eps);
     float *q = y + y_off + (size_t)row * len;
+    const bool vec_params = g_stride == 1 && b_stride == 1 && ((g_off | b_off) & 3u) == 0;
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
-        uint32_t c = (j * WAVE + lane) * 4u;
+        uint32_t c = (j * LPR + li) * 4u;
         if (c < len) {
-            float g[4], b[4];
+            f32x4 g, b;
+            if (vec_params) {
+                g = *reinterpret_cast<const f32x4 *>(gamma + g_off + c);
+                b = *reinterpret_cast<const f32x4 *>(beta + b_off + c);
+            } else {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                g[t] = gamma[g_off + (c + t) * g_stride];
-                b[t] = beta[b_off + (c + t) * b_stride];
+                for (int t = 0; t < 4; ++t) {
+                    g[t] = gamma[g_off + (c + t) * g_stride];
+                    b[t] = beta[b_off + (c + t) * b_stride];
+                }
             }
-            float4 o;
-            o.x = (r.v[j].x - mean) / denom * g[0] + b[0];
-            o.y = (r.v[j].y - mean) / denom * g[1] + b[1];
-            o.z = (r.v[j].z - mean) / denom * g[2] + b[2];
-            o.w = (r.v[j].w - mean) / denom * g[3] + b[3];
-            *reinterpret_cast<float4 *>(q + c) = o;
+            *reinterpret_cast<f32x4 *>(q + c) = (r.v[j] - mean) * inv * g + b;
         }
     }
 }
@@ -511,6 +524,23 @@ int64_t row_dims(const sg_tensor *t, Dims &d) {
 
 }  // namespace
 
+// Rows of up to 256 floats are dealt to 4..64 lanes (one chunk each, several rows per wavefront);
+// longer rows to all 64 lanes with 2..8 chunks per lane.  Expects SG_ROW_LAUNCH(NCHUNK, LPR).
+#define SG_ROW_DISPATCH(LEN)                                                                                            \
+    do {                                                                                                                \
+        const uint32_t len_ = (LEN);                                                                                    \
+        if (len_ <= 16) SG_ROW_LAUNCH(1, 4);                                                                            \
+        else if (len_ <= 32) SG_ROW_LAUNCH(1, 8);                                                                       \
+        else if (len_ <= 64) SG_ROW_LAUNCH(1, 16);                                                                      \
+        else if (len_ <= 128) SG_ROW_LAUNCH(1, 32);                                                                     \
+        else if (len_ <= 256) SG_ROW_LAUNCH(1, 64);                                                                     \
+        else if (len_ <= 512) SG_ROW_LAUNCH(2, 64);                                                                     \
+        else if (len_ <= 768) SG_ROW_LAUNCH(3, 64);                                                                     \
+        else if (len_ <= 1024) SG_ROW_LAUNCH(4, 64);                                                                    \
+        else if (len_ <= 1536) SG_ROW_LAUNCH(6, 64);                                                                    \
+        else SG_ROW_LAUNCH(8, 64);                                                                                      \
+    } while (0)
+
 extern "C" int sg_reduce(sg_ctx *ctx, int op, const int32_t *axes, int n_axes, int init_mode, const sg_tensor *in,
                          const sg_tensor *out) {
     if (!ctx) return SG_ERR_ARG;
@@ -631,23 +661,15 @@ extern "C" int sg_softmax_lastaxis(sg_ctx *ctx, const sg_tensor *x, const sg_ten
     float *yp = (float *)out->base;
     const bool vec = len % 4 == 0 && len <= 2048 && aligned16(x->base, x->offset) && dims_mult4(xo) && aligned16(out->base, out->offset) &&
                      (!addend || ao.inner_stride != 1 || (aligned16(addend->base, addend->offset) && dims_mult4(ao.outer)));
-    dim3 grid((unsigned)((n_rows + 3) / 4));
     if (vec) {
-        const int nchunk = (int)((len + 255) / 256);
-#define SG_SM(NC)                                                                                                       \
+#define SG_ROW_LAUNCH(NC, LPR)                                                                                          \
     do {                                                                                                                \
-        if (addend) hipLaunchKernelGGL((softmax_row_kernel<NC, true>), grid, dim3(256), 0, ctx->stream, xp, ap, yp, (uint32_t)n_rows, len, (uint32_t)x->offset, xo, ao, (uint32_t)out->offset); \
-        else hipLaunchKernelGGL((softmax_row_kernel<NC, false>), grid, dim3(256), 0, ctx->stream, xp, ap, yp, (uint32_t)n_rows, len, (uint32_t)x->offset, xo, ao, (uint32_t)out->offset); \
+        dim3 grid((unsigned)((n_rows + 4 * (64 / LPR) - 1) / (4 * (64 / LPR))));                                        \
+        if (addend) hipLaunchKernelGGL((softmax_row_kernel<NC, LPR, true>), grid, dim3(256), 0, ctx->stream, xp, ap, yp, (uint32_t)n_rows, len, (uint32_t)x->offset, xo, ao, (uint32_t)out->offset); \
+        else hipLaunchKernelGGL((softmax_row_kernel<NC, LPR, false>), grid, dim3(256), 0, ctx->stream, xp, ap, yp, (uint32_t)n_rows, len, (uint32_t)x->offset, xo, ao, (uint32_t)out->offset); \
     } while (0)
-        switch (nchunk) {
-        case 1: SG_SM(1); break;
-        case 2: SG_SM(2); break;
-        case 3: SG_SM(3); break;
-        case 4: SG_SM(4); break;
-        case 5: case 6: SG_SM(6); break;
-        default: SG_SM(8); break;
-        }
-#undef SG_SM
+        SG_ROW_DISPATCH(len);
+#undef SG_ROW_LAUNCH
     } else {
         if (addend) hipLaunchKernelGGL((softmax_row_generic_kernel<true>), dim3((unsigned)n_rows), dim3(256), 0, ctx->stream, xp, ap, yp, len, (uint32_t)x->offset, xo, ao, (uint32_t)out->offset);
         else hipLaunchKernelGGL((softmax_row_generic_kernel<false>), dim3((unsigned)n_rows), dim3(256), 0, ctx->stream, xp, ap, yp, len, (uint32_t)x->offset, xo, ao, (uint32_t)out->offset);
@@ -675,18 +697,13 @@ extern "C" int sg_softmax_cross_entropy(sg_ctx *ctx, const sg_tensor *logits, co
     const uint32_t rs = (uint32_t)logits->strides[0], cs = (uint32_t)logits->strides[1];
     const bool vec = (cs == 1 || C == 1) && C % 4 == 0 && C <= 2048 && aligned16(logits->base, logits->offset) && rs % 4 == 0;
     if (vec) {
-        dim3 grid((unsigned)((B + 3) / 4));
-        const int nchunk = (int)((C + 255) / 256);
-#define SG_CE(NC) hipLaunchKernelGGL((softmax_ce_row_kernel<NC>), grid, dim3(256), 0, ctx->stream, xp, lp, yp, (uint32_t)B, C, (uint32_t)logits->offset, rs, (uint32_t)labels->offset, (uint32_t)labels->strides[0], (uint32_t)loss->offset)
-        switch (nchunk) {
-        case 1: SG_CE(1); break;
-        case 2: SG_CE(2); break;
-        case 3: SG_CE(3); break;
-        case 4: SG_CE(4); break;
-        case 5: case 6: SG_CE(6); break;
-        default: SG_CE(8); break;
-        }
-#undef SG_CE
+#define SG_ROW_LAUNCH(NC, LPR)                                                                                          \
+    do {                                                                                                                \
+        dim3 grid((unsigned)((B + 4 * (64 / LPR) - 1) / (4 * (64 / LPR))));                                             \
+        hipLaunchKernelGGL((softmax_ce_row_kernel<NC, LPR>), grid, dim3(256), 0, ctx->stream, xp, lp, yp, (uint32_t)B, C, (uint32_t)logits->offset, rs, (uint32_t)labels->offset, (uint32_t)labels->strides[0], (uint32_t)loss->offset); \
+    } while (0)
+        SG_ROW_DISPATCH(C);
+#undef SG_ROW_LAUNCH
     } else {
         hipLaunchKernelGGL(softmax_ce_row_generic_kernel, dim3((unsigned)B), dim3(256), 0, ctx->stream, xp, lp, yp, C, (uint32_t)logits->offset, rs, cs,
                            (uint32_t)labels->offset, (uint32_t)labels->strides[0], (uint32_t)loss->offset);
@@ -719,18 +736,13 @@ extern "C" int sg_layer_norm_lastaxis(sg_ctx *ctx, const sg_tensor *x, const sg_
     const uint32_t gs = ng == 1 ? 0u : 1u, bs = nb == 1 ? 0u : 1u;
     const bool vec = len % 4 == 0 && len <= 2048 && aligned16(x->base, x->offset) && dims_mult4(xo) && aligned16(out->base, out->offset);
     if (vec) {
-        dim3 grid((unsigned)((n_rows + 3) / 4));
-        const int nchunk = (int)((len + 255) / 256);
-#define SG_LN(NC) hipLaunchKernelGGL((layer_norm_row_kernel<NC>), grid, dim3(256), 0, ctx->stream, xp, gp, bp, yp, (uint32_t)n_rows, len, (uint32_t)x->offset, xo, (uint32_t)gamma->offset, gs, (uint32_t)beta->offset, bs, eps, (uint32_t)out->offset)
-        switch (nchunk) {
-        case 1: SG_LN(1); break;
-        case 2: SG_LN(2); break;
-        case 3: SG_LN(3); break;
-        case 4: SG_LN(4); break;
-        case 5: case 6: SG_LN(6); break;
-        default: SG_LN(8); break;
-        }
-#undef SG_LN
+#define SG_ROW_LAUNCH(NC, LPR)                                                                                          \
+    do {                                                                                                                \
+        dim3 grid((unsigned)((n_rows + 4 * (64 / LPR) - 1) / (4 * (64 / LPR))));                                        \
+        hipLaunchKernelGGL((layer_norm_row_kernel<NC, LPR>), grid, dim3(256), 0, ctx->stream, xp, gp, bp, yp, (uint32_t)n_rows, len, (uint32_t)x->offset, xo, (uint32_t)gamma->offset, gs, (uint32_t)beta->offset, bs, eps, (uint32_t)out->offset); \
+    } while (0)
+        SG_ROW_DISPATCH(len);
+#undef SG_ROW_LAUNCH
     } else {
         hipLaunchKernelGGL(layer_norm_row_generic_kernel, dim3((unsigned)n_rows), dim3(256), 0, ctx->stream, xp, gp, bp, yp, len, (uint32_t)x->offset, xo,
                            (uint32_t)gamma->offset, gs, (uint32_t)beta->offset, bs, eps, (uint32_t)out->offset);

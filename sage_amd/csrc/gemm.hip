@@ -73,6 +73,10 @@ template <int ROWS, bool K_CONTIG> struct Tile {
     static constexpr int LD = K_CONTIG ? BK + KPAD : ROWS + RPAD;
     static constexpr int SIZE = K_CONTIG ? ROWS * LD : BK * LD;      // floats
 
+    // When the slab does not divide evenly over the threads, the surplus slots of the last round
+    // repeat earlier ones (same element, same value, same LDS address) instead of branching.
+    __device__ static __forceinline__ int slot(int f) { return (TOTAL % NTHREADS == 0 || f < TOTAL) ? f : f - (NV * NTHREADS - TOTAL); }
+
     // element (row, k) of the slab handled by slot f of this thread
     __device__ static __forceinline__ void where(int f, int &row, int &k) {
         if (K_CONTIG) {
@@ -89,13 +93,11 @@ template <int ROWS, bool K_CONTIG> struct Tile {
     __device__ static __forceinline__ void load_fast(f32x4 (&r)[NV], const float *base, int row0, int k0, int64_t s_row, int64_t s_k, int tid) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int f = tid + i * NTHREADS;
-            if (TOTAL % NTHREADS == 0 || f < TOTAL) {
-                int row, k;
-                where(f, row, k);
-                const float *p = K_CONTIG ? base + (int64_t)(row0 + row) * s_row + (k0 + k) : base + (int64_t)(k0 + k) * s_k + (row0 + row);
-                r[i] = *reinterpret_cast<const f32x4 *>(p);
-            }
+            const int f = slot(tid + i * NTHREADS);
+            int row, k;
+            where(f, row, k);
+            const float *p = K_CONTIG ? base + (int64_t)(row0 + row) * s_row + (k0 + k) : base + (int64_t)(k0 + k) * s_k + (row0 + row);
+            r[i] = *reinterpret_cast<const f32x4 *>(p);
         }
     }
 
@@ -104,9 +106,9 @@ template <int ROWS, bool K_CONTIG> struct Tile {
                                                         int64_t s_k, int vec_ok, int tid) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int f = tid + i * NTHREADS;
+            const int f = slot(tid + i * NTHREADS);
             f32x4 v = {0.f, 0.f, 0.f, 0.f};
-            if (TOTAL % NTHREADS == 0 || f < TOTAL) {
+            {
                 int row, k;
                 where(f, row, k);
                 const int gr = row0 + row, gk = k0 + k;
@@ -143,12 +145,10 @@ template <int ROWS, bool K_CONTIG> struct Tile {
     __device__ static __forceinline__ void store(const f32x4 (&r)[NV], float *lds, int tid) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int f = tid + i * NTHREADS;
-            if (TOTAL % NTHREADS == 0 || f < TOTAL) {
-                int row, k;
-                where(f, row, k);
-                *reinterpret_cast<f32x4 *>(&lds[lds_at(row, k)]) = r[i];
-            }
+            const int f = slot(tid + i * NTHREADS);
+            int row, k;
+            where(f, row, k);
+            *reinterpret_cast<f32x4 *>(&lds[lds_at(row, k)]) = r[i];
         }
     }
 
@@ -166,7 +166,7 @@ template <int ROWS, bool K_CONTIG> struct Tile {
 };
 
 template <int BM, int BN, int WAVES_M, bool A_KC, bool B_NC, bool GUARD>
-__global__ void __launch_bounds__(NTHREADS) gemm_mfma_kernel(const GemmP p) {
+__global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3, 8))) gemm_mfma_kernel(const GemmP p) {
     constexpr int WAVES_N = 4 / WAVES_M;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -195,9 +195,9 @@ __global__ void __launch_bounds__(NTHREADS) gemm_mfma_kernel(const GemmP p) {
     const int tile_n = (pid % in_group) / gsize;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-    const int b0 = blockIdx.y / p.nb1, b1 = blockIdx.y % p.nb1;
-    const float *A = p.A + b0 * p.a_sb0 + b1 * p.a_sb1;
-    const float *B = p.B + b0 * p.b_sb0 + b1 * p.b_sb1;
+    const int bt0 = blockIdx.y / p.nb1, bt1 = blockIdx.y % p.nb1;
+    const float *A = p.A + bt0 * p.a_sb0 + bt1 * p.a_sb1;
+    const float *B = p.B + bt0 * p.b_sb0 + bt1 * p.b_sb1;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -210,57 +210,100 @@ __global__ void __launch_bounds__(NTHREADS) gemm_mfma_kernel(const GemmP p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    f32x4 ra[TA::NV], rb[TB::NV];
-#define SG_LOAD_SLAB(k0)                                                                       \
+    // Two register sets for the global fetch: slab s travels through set s&1.
+    f32x4 ra0[TA::NV], rb0[TB::NV], ra1[TA::NV], rb1[TB::NV];
+#define SG_LOAD_SLAB(RA, RB, k0)                                                               \
     do {                                                                                       \
         if (GUARD) {                                                                           \
-            TA::load_guarded(ra, A, m0, (k0), p.M, p.K, p.a_sm, p.a_sk, p.vec_a, tid);              \
-            TB::load_guarded(rb, B, n0, (k0), p.N, p.K, p.b_sn, p.b_sk, p.vec_b, tid);              \
+            TA::load_guarded(RA, A, m0, (k0), p.M, p.K, p.a_sm, p.a_sk, p.vec_a, tid);         \
+            TB::load_guarded(RB, B, n0, (k0), p.N, p.K, p.b_sn, p.b_sk, p.vec_b, tid);         \
         } else {                                                                               \
-            TA::load_fast(ra, A, m0, (k0), p.a_sm, p.a_sk, tid);                                    \
-            TB::load_fast(rb, B, n0, (k0), p.b_sn, p.b_sk, tid);                                    \
+            TA::load_fast(RA, A, m0, (k0), p.a_sm, p.a_sk, tid);                               \
+            TB::load_fast(RB, B, n0, (k0), p.b_sn, p.b_sk, tid);                               \
+        }                                                                                      \
+    } while (0)
+#define SG_FETCH(AS, BS, G, AR, BR)                                                            \
+    do {                                                                                       \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i) TA::fetch(AS, a_col + i * 32, G, khalf, AR[i]); \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j) TB::fetch(BS, b_col + j * 32, G, khalf, BR[j]); \
+    } while (0)
+#define SG_MFMA_GROUP(AR, BR)                                                                  \
+    do {                                                                                       \
+        _Pragma("unroll") for (int s = 0; s < 4; ++s)                                          \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i)                                     \
+                _Pragma("unroll") for (int j = 0; j < TN; ++j)                                 \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(AR[i][s], BR[j][s], acc[i][j], 0, 0, 0); \
+    } while (0)
+
+    // Software pipeline of one wavefront, per K slab of 16 (two groups g0, g1 of four MFMA k-steps):
+    //   S1  issue the LDS reads of this slab's g1 operands
+    //   S2  write slab kt+1 (in registers since iteration kt-2) to the other LDS buffer and request
+    //       slab kt+3 from global memory into the registers just freed
+    //   S3  MFMAs of g0 (operands were read during the previous iteration)
+    //   --  barrier: every wavefront's S2 writes are now visible
+    //   S4  issue the LDS reads of the NEXT slab's g0 operands
+    //   S5  MFMAs of g1
+    // Every LDS read has a whole MFMA group to land, a global fetch has two iterations, and there
+    // is one barrier per slab.  Scheduling hints interleave the memory instructions between MFMAs.
+    // Hazards: S2 overwrites the buffer last read in the previous iteration's S1/S4; a wavefront can
+    // only get there after the previous barrier, which all wavefronts reach after those reads have
+    // returned (lgkmcnt(0) precedes the barrier).  S1 reads what the previous S2 wrote before that
+    // same barrier; S4 reads what this iteration's S2 wrote before this iteration's barrier.
+    static_assert(BK == 16, "the pipeline below is written for two groups of four k-steps per slab");
+    constexpr int NMFMA = 4 * TM * TN;  // MFMAs per group
+    const int a_col = wm * WM + (lane & 31), b_col = wn * WN + (lane & 31), khalf = lane >> 5;
+    float a0[TM][4], b0[TN][4], a1[TM][4], b1[TN][4];
+    // The body is unconditional so that each half of the loop is one scheduling region: past the
+    // end of K the write goes to a buffer nobody reads again and the fetch re-reads the last slab
+    // (unguarded path) or returns zeros (guarded path).  The slab count is rounded up to even; the
+    // unguarded path therefore requires K % 32 == 0, the guarded one multiplies a slab of zeros.
+    const int nk = ((p.K + BK - 1) / BK + 1) & ~1;
+    const int k_last = GUARD ? (nk + 2) * BK : (nk - 1) * BK;
+#define SG_SLAB_BODY(KT, RA, RB)                                                               \
+    do {                                                                                       \
+        const int cur = (KT) & 1;                                                              \
+        SG_FETCH(lds_a[cur], lds_b[cur], 1, a1, b1);                                           \
+        TA::store(RA, lds_a[cur ^ 1], tid);                                                    \
+        TB::store(RB, lds_b[cur ^ 1], tid);                                                    \
+        SG_LOAD_SLAB(RA, RB, min(((KT) + 3) * BK, k_last));                                    \
+        SG_MFMA_GROUP(a0, b0);                                                                 \
+        _Pragma("unroll") for (int q = 0; q < NMFMA - 3; ++q) {                                \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                 \
+        }                                                                                      \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
+        __builtin_amdgcn_sched_group_barrier(0x200, TA::NV + TB::NV, 0);                       \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
+        __builtin_amdgcn_sched_group_barrier(0x020, TA::NV + TB::NV, 0);                       \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
+        __syncthreads();                                                                       \
+        SG_FETCH(lds_a[cur ^ 1], lds_b[cur ^ 1], 0, a0, b0);                                   \
+        SG_MFMA_GROUP(a1, b1);                                                                 \
+        _Pragma("unroll") for (int q = 0; q < NMFMA; ++q) {                                    \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);                                 \
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);                                 \
         }                                                                                      \
     } while (0)
 
-    // LDS is double-buffered: slab kt is multiplied out of buffer kt&1 while slab kt+1 (already in
-    // registers) is written to the other buffer and slab kt+2 is fetched from global memory.
-    const int nk = (p.K + BK - 1) / BK;
-    SG_LOAD_SLAB(0);
-    TA::store(ra, lds_a[0], tid);
-    TB::store(rb, lds_b[0], tid);
-    if (nk > 1) SG_LOAD_SLAB(BK);
+    SG_LOAD_SLAB(ra0, rb0, 0);
+    SG_LOAD_SLAB(ra1, rb1, BK);
+    TA::store(ra0, lds_a[0], tid);
+    TB::store(rb0, lds_b[0], tid);
+    SG_LOAD_SLAB(ra0, rb0, min(2 * BK, k_last));
     __syncthreads();
-
-    const int a_col = wm * WM + (lane & 31), b_col = wn * WN + (lane & 31), khalf = lane >> 5;
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) {
-            TA::store(ra, lds_a[cur ^ 1], tid);
-            TB::store(rb, lds_b[cur ^ 1], tid);
-            if (kt + 2 < nk) SG_LOAD_SLAB((kt + 2) * BK);
-        }
-        const float *as = lds_a[cur], *bs = lds_b[cur];
-#pragma unroll
-        for (int g = 0; g < BK / 8; ++g) {
-            float a[TM][4], b[TN][4];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) TA::fetch(as, a_col + i * 32, g, khalf, a[i]);
-#pragma unroll
-            for (int j = 0; j < TN; ++j) TB::fetch(bs, b_col + j * 32, g, khalf, b[j]);
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
-        }
-        __syncthreads();
+    SG_FETCH(lds_a[0], lds_b[0], 0, a0, b0);
+    for (int kt = 0; kt < nk; kt += 2) {
+        SG_SLAB_BODY(kt, ra1, rb1);
+        SG_SLAB_BODY(kt + 1, ra0, rb0);
     }
-
+#undef SG_SLAB_BODY
 #undef SG_LOAD_SLAB
+#undef SG_FETCH
+#undef SG_MFMA_GROUP
+
     // ---- epilogue: element r of a 32x32 block sits at row (r/4)*8 + (lane/32)*4 + r%4, col lane%32
-    float *C = p.C + b0 * p.c_sb0 + b1 * p.c_sb1;
-    const float *R = p.res ? p.res + b0 * p.r_sb0 + b1 * p.r_sb1 : nullptr;
+    float *C = p.C + bt0 * p.c_sb0 + bt1 * p.c_sb1;
+    const float *R = p.res ? p.res + bt0 * p.r_sb0 + bt1 * p.r_sb1 : nullptr;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int n = n0 + wn * WN + j * 32 + (lane & 31);
@@ -296,7 +339,7 @@ void launch_layouts(sg_ctx *ctx, const GemmP &p, dim3 grid, bool a_kc, bool b_nc
 
 // GUARD = false needs every tile to lie fully inside the matrices and 16-byte loads to be legal.
 bool needs_guard(const GemmP &p, int bm, int bn) {
-    return p.M % bm != 0 || p.N % bn != 0 || p.K % BK != 0 || !p.vec_a || !p.vec_b;
+    return p.M % bm != 0 || p.N % bn != 0 || p.K % (2 * BK) != 0 || !p.vec_a || !p.vec_b;
 }
 
 template <int BM, int BN, int WAVES_M>
@@ -433,7 +476,7 @@ extern "C" int sg_gemm_kernel_name(sg_ctx *ctx, int64_t M, int64_t N, int64_t K,
     if (!ctx || !buf || cap < 8) return SG_ERR_ARG;
     const TileCfg &t = kTileCfgs[choose_tile(ctx->num_cus, (int)M, (int)N, (int)batch)];
     // the fast instantiation when the shape tiles exactly (operands assumed 16-byte aligned here)
-    const bool guard = M % t.bm != 0 || N % t.bn != 0 || K % BK != 0;
+    const bool guard = M % t.bm != 0 || N % t.bn != 0 || K % (2 * BK) != 0;
     snprintf(buf, cap, "gemm_mfma_kernel<%d, %d, %d, %s, %s, %s>", t.bm, t.bn, t.waves_m, a_k_contiguous ? "true" : "false",
              b_n_contiguous ? "true" : "false", guard ? "true" : "false");
     return SG_OK;

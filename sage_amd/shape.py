@@ -186,6 +186,56 @@ class Shape:
         s.extents[axis] = end - start + 1
         return s
 
+    def reshape_view(self, extents):
+        """Strides that present this (possibly non-dense) layout with `extents` without moving data,
+        or None when no such strides exist.  The reference always copies a non-default layout before
+        a reshape (core.rs:213-233); this is the zero-copy case analysis it skips: old axes are
+        grouped into runs that are contiguous among themselves and each run is re-split."""
+        extents = [int(e) for e in extents]
+        n = 1
+        for e in extents:
+            n *= e
+        if n != self.size():
+            return None
+        old = [(e, s) for e, s in zip(self.extents, self.strides) if e != 1]
+        new_strides = [0] * len(extents)
+        oi = 0
+        ni = 0
+        while ni < len(extents):
+            if extents[ni] == 1:
+                new_strides[ni] = 0
+                ni += 1
+                continue
+            if oi >= len(old):
+                return None
+            # take old axes until their product covers a run of new axes
+            op, np_ = old[oi][0], extents[ni]
+            o_start, n_start = oi, ni
+            while op != np_:
+                if op < np_:
+                    oi += 1
+                    if oi >= len(old):
+                        return None
+                    op *= old[oi][0]
+                else:
+                    ni += 1
+                    if ni >= len(extents):
+                        return None
+                    np_ *= extents[ni]
+            # the old axes of this run must be contiguous among themselves
+            for k in range(o_start, oi):
+                if old[k][1] != old[k + 1][1] * old[k + 1][0]:
+                    return None
+            stride = old[oi][1]
+            for k in range(ni, n_start - 1, -1):
+                new_strides[k] = stride
+                stride *= extents[k]
+            oi += 1
+            ni += 1
+        if oi != len(old):
+            return None
+        return Shape(extents, new_strides, self.offset)
+
     def expand(self, extents):
         """shape.rs:239-279: left-pad with (1, stride 0), then mute broadcast axes with stride 0."""
         extents = [int(e) for e in extents]

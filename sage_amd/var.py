@@ -673,6 +673,11 @@ class _Evaluator:
     def _ev_reshape(self, v):
         x = self.get(v.inputs[0])
         if not x.is_dense():
+            # a strided tensor (e.g. a column block of a wider GEMM result) can often be re-viewed
+            # in place; only layouts that really need it are copied (core.rs:213-233 always copies)
+            sh = x.shape.reshape_view(v.extents) if _FUSION["on"] else None
+            if sh is not None:
+                return x.with_shape(sh)
             x = self.run_copy(x)
         return x.with_shape(Shape(v.extents, default_strides(v.extents), x.shape.offset))
 
@@ -1006,6 +1011,10 @@ class _Evaluator:
             for u in self.users.get(id(n), ()):
                 if id(u) not in inside:
                     return None
+        if m["bias"] is not None and m["alpha"] == 1.0 and res is None and "act" not in m and "act_post" not in m:
+            t = self.try_sibling_gemms(v, m)
+            if t is not None:
+                return t
         epi = {"alpha": m["alpha"], "act": m.get("act", abi.ACT_NONE), "act_post": m.get("act_post", abi.ACT_NONE)}
         if m["bias"] is not None:
             bt = self.get(m["bias"])
@@ -1019,6 +1028,113 @@ class _Evaluator:
             epi["res"] = rt.with_shape(Shape(g.extents, default_strides(g.extents), rt.shape.offset))
         y = self.run_gemm(g, epi)
         return y.with_shape(Shape(v.extents, default_strides(v.extents), y.shape.offset))
+
+    # ---- pattern: several Dense layers reading the same activations become one wider GEMM
+    def _dense_chain_above(self, g):
+        """gemm node g -> the `reshape*(g) + expand(bias)` node that is its only consumer chain, or None."""
+        n = g
+        while True:
+            us = self.users.get(id(n), ())
+            if len(us) != 1 or id(n) in self.targets or self.done(n):
+                return None
+            u = us[0]
+            if u.op == "reshape":
+                n = u
+                continue
+            if u.op == "binary" and u.attrs["name"] == "add":
+                return u
+            return None
+
+    def try_sibling_gemms(self, v, m):
+        """Dense layers that share their input (the q/k/v projections, bert.rs:254-256) are the same
+        A times different weight matrices: run them as ONE GEMM against the weights laid side by
+        side, and hand every layer a column block of the result (a strided view, no copy).  The
+        concatenated weights and biases are built once per weight set and kept on the context."""
+        g = m["g"]
+        if g.op != "gemm" or g.attrs["ta"] or g.attrs["tb"]:
+            return None
+        a_node, w_node = g.inputs
+        if w_node.op == "reshape":
+            w_node = w_node.inputs[0]
+        if w_node.op != "data" or m["bias"].op != "data":
+            return None
+        root = a_node
+        while root.op == "reshape":
+            root = root.inputs[0]
+        members = []  # (chain root node, gemm node, weight Var, bias Var)
+        seen = set()
+        for u1 in self.users.get(id(root), ()):
+            cands = [u1] if u1.op == "gemm" else list(self.users.get(id(u1), ())) if u1.op == "reshape" else []
+            for g2 in cands:
+                if id(g2) in seen or g2.op != "gemm" or g2.attrs["ta"] or g2.attrs["tb"] or self.done(g2):
+                    continue
+                a2 = g2.inputs[0]
+                r2 = a2
+                while r2.op == "reshape":
+                    r2 = r2.inputs[0]
+                if r2 is not root or a2.extents != a_node.extents:
+                    continue
+                top = v if g2 is g else self._dense_chain_above(g2)
+                if top is None or self.done(top):
+                    continue
+                sub = []
+                m2 = self._match_core(top, sub)
+                if m2 is None or m2["g"] is not g2 or m2["bias"] is None or m2["alpha"] != 1.0:
+                    continue
+                w2 = g2.inputs[1].inputs[0] if g2.inputs[1].op == "reshape" else g2.inputs[1]
+                if w2.op != "data" or m2["bias"].op != "data" or w2.value is None or m2["bias"].value is None:
+                    continue
+                # every intermediate of the sibling must be private to its chain
+                inside = {id(n) for n in sub} | {id(top)}
+                if any(id(u) not in inside for n in sub if n is not top for u in self.users.get(id(n), ())):
+                    continue
+                seen.add(id(g2))
+                members.append((top, g2, w2, m2["bias"]))
+        if len(members) < 2 or not any(t is v for t, _, _, _ in members):
+            return None
+        members.sort(key=lambda t: id(t[2]))
+        ws = [w.value for _, _, w, _ in members]
+        bs = [b.value for _, _, _, b in members]
+        if not all(w.is_dense() and w.rank == 2 and w.extents[0] == ws[0].extents[0] for w in ws) or not all(b.is_dense() for b in bs):
+            return None
+        key = tuple((w.buf.ptr, w.shape.offset, b.buf.ptr, b.shape.offset) for w, b in zip(ws, bs))
+        cache = self.ctx.__dict__.setdefault("_wide_weights", {})
+        if key not in cache:
+            K = ws[0].extents[0]
+            ntot = sum(w.extents[1] for w in ws)
+            wcat, bcat = self.out([K, ntot], FLOAT), self.out([ntot], FLOAT)
+            wi = (abi.sg_tensor * len(ws))(*[w.c() for w in ws])
+            wc = wcat.c()
+            self.ctx.check(self.lib.sg_concat(self.ctx.handle, 1, wi, len(ws), C.byref(wc)))
+            bi = (abi.sg_tensor * len(bs))(*[b.with_shape(Shape([b.size()], [1], b.shape.offset)).c() for b in bs])
+            bc = bcat.c()
+            self.ctx.check(self.lib.sg_concat(self.ctx.handle, 0, bi, len(bs), C.byref(bc)))
+            cache[key] = (wcat, bcat, ws, bs)  # the sources are kept so their pointers stay unique
+        wcat, bcat = cache[key][0], cache[key][1]
+        a = self.get(a_node)
+        if not a.is_dense():
+            a = self.run_copy(a)
+        M, ntot = a.extents[0], wcat.extents[1]
+        y = self.out([M, ntot], FLOAT)
+        epi = {"alpha": 1.0, "bias": bcat}
+        keep = self.keepalive
+        e = self._epi_struct(epi, keep)
+        keep.append(e)
+        ac, wc, yc = a.c(), wcat.c(), y.c()
+        self.call(self.lib.sg_gemm, 0, 0, C.byref(ac), C.byref(wc), C.byref(yc), C.byref(e))
+        off, mine = 0, None
+        for top, g2, w2, _ in members:
+            n = w2.value.extents[1]
+            blk = y.with_shape(Shape([M, n], [ntot, 1], y.shape.offset + off))
+            sh = blk.shape.reshape_view(top.extents)
+            t = blk.with_shape(sh) if sh is not None else self.run_copy(blk).with_shape(Shape(top.extents))
+            off += n
+            if top is v:
+                mine = t
+            else:
+                self.memo[id(top)] = t
+                self.keep[id(top)] = top
+        return mine
 
     def _match_res(self, v, chain):
         """(act?(core)) + R  in either order."""

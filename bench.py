@@ -27,6 +27,19 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
 
+def measured_traffic(kernel, workload):
+    """HBM bytes per dispatch of `kernel` from the committed rocprofv3 counter summary of this same
+    workload (profiles/traffic_<workload>.json: FETCH_SIZE and WRITE_SIZE runs scaled by a copy kernel
+    of known size), or None when there is no such measurement."""
+    path = os.path.join(ROOT, "profiles", f"traffic_{workload}.json")
+    try:
+        with open(path) as f:
+            k = json.load(f)["kernels"].get(kernel)
+        return k["traffic_bytes_per_dispatch"] if k else None
+    except (OSError, ValueError, KeyError):
+        return None
+
+
 def build_bert(ctx, variant, batch, seq, layers, rng):
     import sage_amd as S
     from sage_amd.bert import Bert, BertConfig
@@ -339,7 +352,9 @@ def main():
                    "hidden": cfg.embed_dim, "heads": cfg.num_attention_heads, "ffn": cfg.hidden_dim, "vocab": cfg.num_vocabs,
                    "launches_per_step": len(prog.calls), "gemm_tflops_whole_step": total_gemm_flops / (ms_per_step * 1e-3) / 1e12},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None, "kernel": dom,
+                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+                     "traffic": measured_traffic(dom, f"bert_base_b{a.batch}_s{a.seq}") if a.layers == 12 and a.variant == "config" else None,
+                     "kernel": dom,
                      "launches_per_step": len(by_name[dom]), "avg_launch_ms": avg_ms, "flops_per_launch": flops_per_launch,
                      "shapes_mnkb": sorted({s for _, _, s in by_name[dom]})},
     }

@@ -66,6 +66,51 @@ def build_bert(ctx, variant, batch, seq, layers, rng):
     return cfg, model, logits
 
 
+def build_resnet18(ctx, batch, rng):
+    """ResNet-18 on [batch, 28, 28, 1] images (the reference's MNIST example shape), Kaiming-normal filters."""
+    import sage_amd as S
+    from sage_amd.resnet import ResNet, ResNetConfig
+    model = ResNet(ResNetConfig.d18(1, 10))
+    arrays = []
+    for p in model.params():
+        ext = p.extents
+        if len(ext) == 1:
+            a = np.zeros(ext, np.float32)
+        elif len(ext) == 4:
+            a = (rng.standard_normal(ext) * np.sqrt(2.0 / (ext[0] * ext[1] * ext[2]))).astype(np.float32)
+        else:
+            a = (rng.standard_normal(ext) * 0.05).astype(np.float32)
+        arrays.append(a)
+        p.set(S.Tensor.from_numpy(ctx, a))
+    x = rng.uniform(0, 1, (batch, 28, 28, 1)).astype(np.float32)
+    return model, arrays, x, model.pass_(S.Var.new(S.Tensor.from_numpy(ctx, x)))
+
+
+def cpu_baseline_resnet18(model, arrays, x):
+    """The CPU oracle on the whole ResNet-18 forward pass at the bench's batch."""
+    from oracle import oracle as O
+    ht = O.HT.from_numpy
+    it = iter(arrays)
+    pod = {"w0": ht(next(it)), "b0": ht(next(it)), "blocks": []}
+    inp, out = 64, 64
+    for i in range(4):
+        ip = inp
+        for b in range(2):
+            s = (1 if i == 0 else 2) if b == 0 else 1
+            blk = {"stride": s, "w1": ht(next(it)), "b1": ht(next(it)), "w2": ht(next(it)), "b2": ht(next(it))}
+            if s != 1 or ip != out:
+                blk["wd"], blk["bd"] = ht(next(it)), ht(next(it))
+            pod["blocks"].append(blk)
+            ip = out
+        inp, out = out, out * 2
+    pod["wfc"], pod["bfc"] = ht(next(it)), ht(next(it))
+    t0 = time.perf_counter()
+    O.resnet18_forward(ht(x), pod)
+    dt = time.perf_counter() - t0
+    return {"value": x.shape[0] / dt, "unit": "images/s", "cores": O.num_threads(), "kind": "port",
+            "sample": f"one whole forward pass at b{x.shape[0]} in {dt:.2f} s"}
+
+
 def gemm_calls(ctx, prog):
     """(call index, kernel name, flops) for every GEMM launch of the compiled program."""
     from sage_amd import abi
@@ -116,7 +161,8 @@ def run_timed(ctx, prog, timed):
 
 def cpu_baseline(variant, batch, seq, rng_seed):
     """The CPU oracle (oracle/: C restatement of the reference kernels, OpenMP over work-items) on one
-    of the 12 encoder layers at the full b32 x s128 shape; the layer time x 12 gives seqs/s."""
+    of the 12 encoder layers (whole batch at b32 x s128; at most 4096 tokens of it for larger shapes);
+    the layer time x 12 gives seqs/s."""
     from oracle import oracle as O
     rng = np.random.default_rng(rng_seed)
     e, hdim, heads = 768, 3072, 12
@@ -126,6 +172,7 @@ def cpu_baseline(variant, batch, seq, rng_seed):
     one = lambda: O.HT.from_numpy(np.ones(nln, np.float32))
     p = {"wq": w(e, e), "bq": z(e), "wk": w(e, e), "bk": z(e), "wv": w(e, e), "bv": z(e), "wo": w(e, e), "bo": z(e),
          "ln1_g": one(), "ln1_b": z(nln), "w1": w(e, hdim), "b1": z(hdim), "w2": w(hdim, e), "b2": z(e), "ln2_g": one(), "ln2_b": z(nln)}
+    batch = max(1, min(batch, 4096 // seq))  # bounded sample: at most 4096 tokens
     x = O.HT.from_numpy(rng.standard_normal((batch, seq, e)).astype(np.float32))
     mask = O.HT.from_numpy(np.ones((batch, seq), np.float32))
     act, eps = ("relu", 1e-5) if variant == "reference" else ("gelu", 1e-12)
@@ -277,7 +324,7 @@ def run_kernel_workload(a):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="bert", help="bert (default, the headline metric) | softmax_ce | map_exp_sub | "
+    ap.add_argument("--workload", default="bert", help="bert (default, the headline metric) | resnet18 | softmax_ce | map_exp_sub | "
                     "bias_residual | layer_norm | softmax | reduce_sum | gemm_bias")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
@@ -292,7 +339,7 @@ def main():
         print("bench.py measures one GPU: every box in this run has one MI355X and the hot path uses no "
               "collectives; run with --gpus 1", file=sys.stderr)
         sys.exit(2)
-    if a.workload != "bert":
+    if a.workload not in ("bert", "resnet18"):
         return run_kernel_workload(a)
 
     import sage_amd as S
@@ -300,7 +347,12 @@ def main():
     lib = abi.lib()
     ctx = S.Context(0)
     rng = np.random.default_rng(5)
-    cfg, model, logits = build_bert(ctx, a.variant, a.batch, a.seq, a.layers, rng)
+    if a.workload == "resnet18":
+        batch = a.batch if a.batch != 32 else 128
+        model, arrays, x_host, logits = build_resnet18(ctx, batch, rng)
+    else:
+        batch = a.batch
+        cfg, model, logits = build_bert(ctx, a.variant, a.batch, a.seq, a.layers, rng)
     prog = S.Program(ctx, [logits])  # first evaluation: builds kernels, allocates every buffer
     ctx.sync()
     out0 = prog.outputs[0].numpy()
@@ -341,25 +393,31 @@ def main():
     avg_ms = float(np.mean(kernel_ms))
     achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
     total_gemm_flops = sum(f for _, _, f, _ in gc)
+    if a.workload == "resnet18":
+        metric, unit = f"ResNet-18 fwd images/sec (b{batch},28x28x1,fp32)", "images/s"
+        config = {"workload": f"resnet18_forward_b{batch}_28x28x1_fp32"}
+    else:
+        metric, unit = f"BERT-base fwd seqs/sec (b{a.batch},s{a.seq},fp32)", "seqs/s"
+        config = {"workload": f"bert_base_forward_b{a.batch}_s{a.seq}_fp32", "variant": a.variant, "layers": a.layers,
+                  "hidden": cfg.embed_dim, "heads": cfg.num_attention_heads, "ffn": cfg.hidden_dim, "vocab": cfg.num_vocabs}
+    config.update({"launches_per_step": len(prog.calls), "gemm_tflops_whole_step": total_gemm_flops / (ms_per_step * 1e-3) / 1e12})
     res = {
-        "metric": "BERT-base fwd seqs/sec (b32,s128,fp32)",
-        "value": a.batch / (ms_per_step * 1e-3),
-        "unit": "seqs/s",
+        "metric": metric,
+        "value": batch / (ms_per_step * 1e-3),
+        "unit": unit,
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"bert_base_forward_b{a.batch}_s{a.seq}_fp32", "variant": a.variant, "layers": a.layers,
-                   "hidden": cfg.embed_dim, "heads": cfg.num_attention_heads, "ffn": cfg.hidden_dim, "vocab": cfg.num_vocabs,
-                   "launches_per_step": len(prog.calls), "gemm_tflops_whole_step": total_gemm_flops / (ms_per_step * 1e-3) / 1e12},
+        "config": config,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
-                     "traffic": measured_traffic(dom, f"bert_base_b{a.batch}_s{a.seq}") if a.layers == 12 and a.variant == "config" else None,
+                     "traffic": measured_traffic(dom, f"bert_base_b{a.batch}_s{a.seq}") if a.workload == "bert" and a.layers == 12 and a.variant == "config" else None,
                      "kernel": dom,
                      "launches_per_step": len(by_name[dom]), "avg_launch_ms": avg_ms, "flops_per_launch": flops_per_launch,
                      "shapes_mnkb": sorted({s for _, _, s in by_name[dom]})},
     }
     if not a.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline(a.variant, a.batch, a.seq, 6)
+        res["cpu_baseline"] = cpu_baseline_resnet18(model, arrays, x_host) if a.workload == "resnet18" else cpu_baseline(a.variant, a.batch, a.seq, 6)
     print(json.dumps(res))
 
 

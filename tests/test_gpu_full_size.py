@@ -1,0 +1,139 @@
+"""The five benchmark configurations at their full sizes.
+
+Where the CPU oracle finishes in seconds the whole result is compared with it; where it would not,
+size-independent properties are used instead: sampled entries against float64 dot products,
+a row block against the oracle, and batch-slice invariance (the first sequences of a full batch must
+equal a run on just those sequences, which the oracle can check)."""
+import numpy as np
+import pytest
+
+import sage_amd as S
+from oracle import oracle as O
+from sage_amd import nn
+from sage_amd import var as V
+from sage_amd.bert import BertConfig, BertLayer
+from sage_amd.layers import load_params
+from sage_amd.resnet import ResNet, ResNetConfig
+from tests.test_gpu_models import bert_layer_params, layer_param_list, resnet_arrays
+from tests.util import REL_GEMM, REL_MAP, close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = S.Context()
+    yield c
+    c.close()
+
+
+@pytest.fixture(autouse=True)
+def _fusion_on():
+    V.set_fusion(True)
+    yield
+    V.set_fusion(True)
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+
+
+def dev(ctx, a):
+    return S.Var.new(S.Tensor.from_numpy(ctx, a))
+
+
+def ht(a):
+    return O.HT.from_numpy(a)
+
+
+def test_config1_softmax_cross_entropy_8192x1024(ctx):
+    say("C1 softmax-CE [8192,1024]")
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((8192, 1024)).astype(np.float32)
+    lab = rng.integers(0, 1024, (8192, 1)).astype(np.int32)
+    y = nn.softmax_cross_entropy(dev(ctx, x), dev(ctx, lab)).eval(ctx).numpy()
+    x64 = x.astype(np.float64)
+    ref = -(x64[np.arange(8192), lab[:, 0]] - np.log(np.exp(x64).sum(1)))
+    close(y, ref, REL_MAP, "fused vs float64")
+    close(y, O.softmax_cross_entropy(ht(x), ht(lab.astype(np.uint32))).numpy(), REL_MAP, "fused vs oracle")
+    V.set_fusion(False)
+    close(nn.softmax_cross_entropy(dev(ctx, x), dev(ctx, lab)).eval(ctx).numpy(), ref, REL_MAP, "composed vs float64")
+    assert np.all(y >= 0)
+
+
+def test_config2_gemm_4096_bias(ctx):
+    say("C2 GEMM 4096^3 + bias")
+    rng = np.random.default_rng(2)
+    n = 4096
+    a = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    b = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (n,)).astype(np.float32)
+    n0 = ctx.launches
+    y = (dev(ctx, a).matmul(dev(ctx, b)) + dev(ctx, bias)).eval(ctx).numpy()
+    assert ctx.launches - n0 == 1
+    ii, jj = rng.integers(0, n, 512), rng.integers(0, n, 512)
+    ref = np.einsum("ik,ki->i", a[ii].astype(np.float64), b[:, jj].astype(np.float64)) + bias[jj]
+    close(y[ii, jj], ref, REL_GEMM, "sampled entries vs float64")
+    rows = np.arange(1000, 1016)
+    close(y[rows], O.dense(ht(a[rows]), ht(b), ht(bias)).numpy(), REL_GEMM, "16-row block vs oracle")
+    # a checksum of checksums: sum_j C[i,j] = A[i,:] . (B 1) + sum(bias)
+    close(y.astype(np.float64).sum(1), a.astype(np.float64) @ b.astype(np.float64).sum(1) + bias.astype(np.float64).sum(), REL_GEMM, "row checksums")
+
+
+@pytest.mark.parametrize("reference_exact", [True, False], ids=["reference_exact", "gelu_config"])
+def test_config3_bert_layer_b32_s128(ctx, reference_exact):
+    say("C3 BERT layer b32 s128 h768", reference_exact)
+    rng = np.random.default_rng(3)
+    n, l, e, heads, hdim = 32, 128, 768, 12, 3072
+    p = bert_layer_params(rng, e, hdim, per_feature=not reference_exact)
+    for k in p:
+        if k.startswith("w"):
+            p[k] = (p[k] * 0.4).astype(np.float32)  # ~N(0, 0.02)
+    x = rng.standard_normal((n, l, e)).astype(np.float32)
+    mask = np.ones((n, l), np.float32)
+    layer = BertLayer(BertConfig(e, 100, 512, hdim, 1, heads, 1e-12, 0.1, 2), reference_exact)
+    load_params(ctx, layer, layer_param_list(p))
+    n0 = ctx.launches
+    y = layer.pass_(dev(ctx, x), dev(ctx, mask)).eval(ctx).numpy()
+    say("launches", ctx.launches - n0)
+    act, eps = ("relu", 1e-5) if reference_exact else ("gelu", 1e-12)
+    yo = O.bert_layer(ht(x), ht(mask), {k: ht(v) for k, v in p.items()}, heads, act, eps).numpy()
+    close(y, yo, REL_GEMM, "vs oracle")
+
+
+def test_config4_resnet18_b128(ctx):
+    say("C4 ResNet-18 b128 28x28x1")
+    rng = np.random.default_rng(4)
+    arrays, po = resnet_arrays(rng, 1, 10)
+    model = ResNet(ResNetConfig.d18(1, 10))
+    load_params(ctx, model, arrays)
+    x = rng.uniform(0, 1, (128, 28, 28, 1)).astype(np.float32)
+    y = model.pass_(dev(ctx, x)).eval(ctx).numpy()
+    conv = lambda d: {k: (ht(v) if isinstance(v, np.ndarray) else v) for k, v in d.items()}
+    pod = {"w0": ht(po["w0"]), "b0": ht(po["b0"]), "blocks": [conv(b) for b in po["blocks"]], "wfc": ht(po["wfc"]), "bfc": ht(po["bfc"])}
+    close(y, O.resnet18_forward(ht(x), pod).numpy(), REL_GEMM, "vs oracle")
+
+
+def test_config5_bert_layer_b64_s512_batch_slice(ctx):
+    say("C5 BERT layer b64 s512: first 2 sequences of the full batch == a batch of 2 == oracle")
+    rng = np.random.default_rng(5)
+    n, l, e, heads, hdim = 64, 512, 768, 12, 3072
+    p = bert_layer_params(rng, e, hdim, per_feature=True)
+    for k in p:
+        if k.startswith("w"):
+            p[k] = (p[k] * 0.4).astype(np.float32)
+    x = rng.standard_normal((n, l, e)).astype(np.float32)
+    mask = np.ones((n, l), np.float32)
+    mask[1, 400:] = 0.0
+    layer = BertLayer(BertConfig(e, 100, 512, hdim, 1, heads, 1e-12, 0.1, 2), reference_exact=False)
+    load_params(ctx, layer, layer_param_list(p))
+    y_full = layer.pass_(dev(ctx, x), dev(ctx, mask)).eval(ctx).numpy()
+    y_two = layer.pass_(dev(ctx, x[:2]), dev(ctx, mask[:2])).eval(ctx).numpy()
+    close(y_full[:2], y_two, REL_GEMM, "batch-slice invariance")
+    yo = O.bert_layer(ht(x[:2]), ht(mask[:2]), {k: ht(v) for k, v in p.items()}, heads, "gelu", 1e-12).numpy()
+    close(y_two, yo, REL_GEMM, "batch of 2 vs oracle")
+    assert np.all(np.isfinite(y_full))
+    # the layer ends in a layer norm: undoing its affine part leaves rows of mean 0 and variance 1
+    z = (y_full.astype(np.float64) - p["ln2_b"]) / p["ln2_g"]
+    assert np.abs(z.mean(-1)).max() < 1e-3
+    close(z.var(-1), np.ones(z.shape[:2]), REL_GEMM, "rows normalised")

@@ -23,8 +23,9 @@
 //     all; only edge shapes pay for guarded, zero-filling loads.
 //   * Workgroup ids are remapped so that the ids one XCD receives (id mod 8) cover a compact block
 //     of tiles, which keeps the A/B panels a tile group shares inside that XCD's L2.
-//   * The epilogue applies alpha, bias[n], activation and a residual while the accumulators are
-//     still in registers.
+//   * The epilogue applies alpha, bias[n], activation and a residual on the way out: accumulator
+//     blocks go through a per-wavefront LDS stage and leave as 16-byte row segments, in a rolled
+//     loop that keeps the kernel's code small.
 // Accumulation order differs from the reference's sequential k (MFMA sums pairs of k, slabs in
 // order); the difference is fp32 rounding only and is covered by the 1e-3 GEMM tolerance.
 #include "common.h"
@@ -52,6 +53,7 @@ struct GemmP {
     float alpha;
     int act, act_post;
     int vec_a, vec_b;  // 16-byte loads are legal for this operand
+    int vec_c, vec_r, vec_bias;  // 16-byte accesses are legal for C rows / residual rows / the bias
 };
 
 __device__ __forceinline__ float apply_act(float v, int act) {
@@ -89,67 +91,57 @@ template <int ROWS, bool K_CONTIG> struct Tile {
     }
     __device__ static __forceinline__ int lds_at(int row, int k) { return K_CONTIG ? row * LD + k : k * LD + row; }
 
-    // unguarded: whole tile inside the matrix, 16-byte aligned
-    __device__ static __forceinline__ void load_fast(f32x4 (&r)[NV], const float *base, int row0, int k0, int64_t s_row, int64_t s_k, int tid) {
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int f = slot(tid + i * NTHREADS);
-            int row, k;
-            where(f, row, k);
-            const float *p = K_CONTIG ? base + (int64_t)(row0 + row) * s_row + (k0 + k) : base + (int64_t)(k0 + k) * s_k + (row0 + row);
-            r[i] = *reinterpret_cast<const f32x4 *>(p);
-        }
+    // One 16-byte item of the slab (slot i of this thread), unguarded: the whole tile lies inside
+    // the matrix and is 16-byte aligned.
+    __device__ static __forceinline__ void load_one_fast(f32x4 &r, int i, const float *base, int row0, int k0, int64_t s_row, int64_t s_k, int tid) {
+        const int f = slot(tid + i * NTHREADS);
+        int row, k;
+        where(f, row, k);
+        const float *p = K_CONTIG ? base + (int64_t)(row0 + row) * s_row + (k0 + k) : base + (int64_t)(k0 + k) * s_k + (row0 + row);
+        r = *reinterpret_cast<const f32x4 *>(p);
     }
 
     // guarded: zero-fill outside [row_lim) x [k_lim), scalar loads when 16-byte loads are not legal
-    __device__ static __forceinline__ void load_guarded(f32x4 (&r)[NV], const float *base, int row0, int k0, int row_lim, int k_lim, int64_t s_row,
-                                                        int64_t s_k, int vec_ok, int tid) {
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int f = slot(tid + i * NTHREADS);
-            f32x4 v = {0.f, 0.f, 0.f, 0.f};
-            {
-                int row, k;
-                where(f, row, k);
-                const int gr = row0 + row, gk = k0 + k;
-                if (K_CONTIG) {
-                    if (gr < row_lim) {
-                        const float *p = base + (int64_t)gr * s_row + gk;
-                        if (vec_ok && gk + 3 < k_lim) {
-                            v = *reinterpret_cast<const f32x4 *>(p);
-                        } else {
-                            if (gk + 0 < k_lim) v.x = p[0];
-                            if (gk + 1 < k_lim) v.y = p[1];
-                            if (gk + 2 < k_lim) v.z = p[2];
-                            if (gk + 3 < k_lim) v.w = p[3];
-                        }
-                    }
+    __device__ static __forceinline__ void load_one_guarded(f32x4 &r, int i, const float *base, int row0, int k0, int row_lim, int k_lim, int64_t s_row,
+                                                            int64_t s_k, int vec_ok, int tid) {
+        const int f = slot(tid + i * NTHREADS);
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        int row, k;
+        where(f, row, k);
+        const int gr = row0 + row, gk = k0 + k;
+        if (K_CONTIG) {
+            if (gr < row_lim) {
+                const float *p = base + (int64_t)gr * s_row + gk;
+                if (vec_ok && gk + 3 < k_lim) {
+                    v = *reinterpret_cast<const f32x4 *>(p);
                 } else {
-                    if (gk < k_lim) {
-                        const float *p = base + (int64_t)gk * s_k + gr;
-                        if (vec_ok && gr + 3 < row_lim) {
-                            v = *reinterpret_cast<const f32x4 *>(p);
-                        } else {
-                            if (gr + 0 < row_lim) v.x = p[0];
-                            if (gr + 1 < row_lim) v.y = p[1];
-                            if (gr + 2 < row_lim) v.z = p[2];
-                            if (gr + 3 < row_lim) v.w = p[3];
-                        }
-                    }
+                    if (gk + 0 < k_lim) v.x = p[0];
+                    if (gk + 1 < k_lim) v.y = p[1];
+                    if (gk + 2 < k_lim) v.z = p[2];
+                    if (gk + 3 < k_lim) v.w = p[3];
                 }
             }
-            r[i] = v;
+        } else {
+            if (gk < k_lim) {
+                const float *p = base + (int64_t)gk * s_k + gr;
+                if (vec_ok && gr + 3 < row_lim) {
+                    v = *reinterpret_cast<const f32x4 *>(p);
+                } else {
+                    if (gr + 0 < row_lim) v.x = p[0];
+                    if (gr + 1 < row_lim) v.y = p[1];
+                    if (gr + 2 < row_lim) v.z = p[2];
+                    if (gr + 3 < row_lim) v.w = p[3];
+                }
+            }
         }
+        r = v;
     }
 
-    __device__ static __forceinline__ void store(const f32x4 (&r)[NV], float *lds, int tid) {
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int f = slot(tid + i * NTHREADS);
-            int row, k;
-            where(f, row, k);
-            *reinterpret_cast<f32x4 *>(&lds[lds_at(row, k)]) = r[i];
-        }
+    __device__ static __forceinline__ void store_one(const f32x4 &r, int i, float *lds, int tid) {
+        const int f = slot(tid + i * NTHREADS);
+        int row, k;
+        where(f, row, k);
+        *reinterpret_cast<f32x4 *>(&lds[lds_at(row, k)]) = r;
     }
 
     // MFMA operands of one group of 4 k-steps for the 32 rows starting at `col0`: step s of group g
@@ -173,8 +165,13 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA block");
     typedef Tile<BM, A_KC> TA;
     typedef Tile<BN, !B_NC> TB;
-    __shared__ __attribute__((aligned(16))) float lds_a[2][TA::SIZE];
-    __shared__ __attribute__((aligned(16))) float lds_b[2][TB::SIZE];
+    // Operand buffers during the K loop; afterwards the same memory stages the output blocks.
+    constexpr int STAGE_LD = 36, STAGE = 32 * STAGE_LD;  // one 32x32 block per wavefront, padded rows
+    constexpr int LDS_OPERANDS = 2 * TA::SIZE + 2 * TB::SIZE;
+    constexpr int LDS_FLOATS = LDS_OPERANDS > 4 * STAGE ? LDS_OPERANDS : 4 * STAGE;
+    __shared__ __attribute__((aligned(16))) float lds_raw[LDS_FLOATS];
+    float(*lds_a)[TA::SIZE] = reinterpret_cast<float(*)[TA::SIZE]>(lds_raw);
+    float(*lds_b)[TB::SIZE] = reinterpret_cast<float(*)[TB::SIZE]>(lds_raw + 2 * TA::SIZE);
 
     // ---- which tile: spread consecutive ids over XCDs, then walk tiles in groups of 8 tile-rows
     const int ntiles = p.tiles_m * p.tiles_n;
@@ -212,119 +209,192 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
 
     // Two register sets for the global fetch: slab s travels through set s&1.
     f32x4 ra0[TA::NV], rb0[TB::NV], ra1[TA::NV], rb1[TB::NV];
-#define SG_LOAD_SLAB(RA, RB, k0)                                                               \
+    constexpr int NWR = TA::NV + TB::NV;  // 16-byte items per thread and slab (global loads = LDS writes)
+    constexpr int NRB = TM + TN;          // operand fetches (one per 32-row block) per group of k-steps
+    constexpr int NMFMA = 4 * TM * TN;    // MFMAs per group
+    const int a_col = wm * WM + (lane & 31), b_col = wn * WN + (lane & 31), khalf = lane >> 5;
+    float a0[TM][4], b0[TN][4], a1[TM][4], b1[TN][4];
+
+    // item e of a slab: global memory -> registers
+#define SG_ITEM_LOAD(e, RA, RB, k0)                                                            \
     do {                                                                                       \
-        if (GUARD) {                                                                           \
-            TA::load_guarded(RA, A, m0, (k0), p.M, p.K, p.a_sm, p.a_sk, p.vec_a, tid);         \
-            TB::load_guarded(RB, B, n0, (k0), p.N, p.K, p.b_sn, p.b_sk, p.vec_b, tid);         \
+        if ((e) < TA::NV) {                                                                    \
+            const int ia = (e) < TA::NV ? (e) : 0;                                         \
+            if (GUARD) TA::load_one_guarded(RA[ia], ia, A, m0, (k0), p.M, p.K, p.a_sm, p.a_sk, p.vec_a, tid); \
+            else TA::load_one_fast(RA[ia], ia, A, m0, (k0), p.a_sm, p.a_sk, tid);             \
         } else {                                                                               \
-            TA::load_fast(RA, A, m0, (k0), p.a_sm, p.a_sk, tid);                               \
-            TB::load_fast(RB, B, n0, (k0), p.b_sn, p.b_sk, tid);                               \
+            const int ib = (e) >= TA::NV ? (e) - TA::NV : 0;                               \
+            if (GUARD) TB::load_one_guarded(RB[ib], ib, B, n0, (k0), p.N, p.K, p.b_sn, p.b_sk, p.vec_b, tid); \
+            else TB::load_one_fast(RB[ib], ib, B, n0, (k0), p.b_sn, p.b_sk, tid);             \
         }                                                                                      \
     } while (0)
-#define SG_FETCH(AS, BS, G, AR, BR)                                                            \
+    // item e of a slab: registers -> LDS buffer BUF
+#define SG_ITEM_STORE(e, RA, RB, BUF)                                                          \
     do {                                                                                       \
-        _Pragma("unroll") for (int i = 0; i < TM; ++i) TA::fetch(AS, a_col + i * 32, G, khalf, AR[i]); \
-        _Pragma("unroll") for (int j = 0; j < TN; ++j) TB::fetch(BS, b_col + j * 32, G, khalf, BR[j]); \
+        if ((e) < TA::NV) {                                                                    \
+            const int ia = (e) < TA::NV ? (e) : 0;                                         \
+            TA::store_one(RA[ia], ia, lds_a[BUF], tid);                                        \
+        } else {                                                                               \
+            const int ib = (e) >= TA::NV ? (e) - TA::NV : 0;                               \
+            TB::store_one(RB[ib], ib, lds_b[BUF], tid);                                        \
+        }                                                                                      \
     } while (0)
-#define SG_MFMA_GROUP(AR, BR)                                                                  \
+    // fetch e of a group: LDS buffer BUF -> MFMA operand registers of group G
+#define SG_ITEM_FETCH(e, BUF, G, AR, BR)                                                       \
     do {                                                                                       \
-        _Pragma("unroll") for (int s = 0; s < 4; ++s)                                          \
-            _Pragma("unroll") for (int i = 0; i < TM; ++i)                                     \
-                _Pragma("unroll") for (int j = 0; j < TN; ++j)                                 \
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(AR[i][s], BR[j][s], acc[i][j], 0, 0, 0); \
+        if ((e) < TM) {                                                                        \
+            const int ia = (e) < TM ? (e) : 0;                                             \
+            TA::fetch(lds_a[BUF], a_col + ia * 32, G, khalf, AR[ia]);                          \
+        } else {                                                                               \
+            const int ib = (e) >= TM ? (e) - TM : 0;                                       \
+            TB::fetch(lds_b[BUF], b_col + ib * 32, G, khalf, BR[ib]);                          \
+        }                                                                                      \
+    } while (0)
+#define SG_MFMA(t, AR, BR)                                                                     \
+    do {                                                                                       \
+        const int s_ = (t) / (TM * TN), i_ = ((t) / TN) % TM, j_ = (t) % TN;               \
+        acc[i_][j_] = __builtin_amdgcn_mfma_f32_32x32x2f32(AR[i_][s_], BR[j_][s_], acc[i_][j_], 0, 0, 0); \
     } while (0)
 
     // Software pipeline of one wavefront, per K slab of 16 (two groups g0, g1 of four MFMA k-steps):
-    //   S1  issue the LDS reads of this slab's g1 operands
-    //   S2  write slab kt+1 (in registers since iteration kt-2) to the other LDS buffer and request
-    //       slab kt+3 from global memory into the registers just freed
-    //   S3  MFMAs of g0 (operands were read during the previous iteration)
-    //   --  barrier: every wavefront's S2 writes are now visible
-    //   S4  issue the LDS reads of the NEXT slab's g0 operands
-    //   S5  MFMAs of g1
+    //   S3  MFMAs of g0 (operands were read during the previous iteration); behind the first of
+    //       them, in this order: the LDS writes of slab kt+1 (in registers since iteration kt-2)
+    //       to the other buffer, the LDS reads of this slab's g1 operands, and the global requests
+    //       for slab kt+3 into the registers just freed
+    //   --  barrier: every wavefront's writes are now visible
+    //   S5  MFMAs of g1; behind the first of them the LDS reads of the NEXT slab's g0 operands
+    // The instruction order is pinned (scheduling barriers between the steps): memory instructions
+    // issue in the shadow of a running MFMA, the LDS queue drains during the item-free tail of each
+    // group, and the waits in front of the barrier and in front of the next group find it empty.
     // Every LDS read has a whole MFMA group to land, a global fetch has two iterations, and there
-    // is one barrier per slab.  Scheduling hints interleave the memory instructions between MFMAs.
-    // Hazards: S2 overwrites the buffer last read in the previous iteration's S1/S4; a wavefront can
+    // is one barrier per slab.
+    // Hazards: the writes overwrite the buffer last read in the previous iteration; a wavefront can
     // only get there after the previous barrier, which all wavefronts reach after those reads have
-    // returned (lgkmcnt(0) precedes the barrier).  S1 reads what the previous S2 wrote before that
-    // same barrier; S4 reads what this iteration's S2 wrote before this iteration's barrier.
+    // returned (lgkmcnt(0) precedes the barrier).  The g1 reads see what the previous iteration
+    // wrote before that same barrier; the g0 reads see what this iteration wrote before its barrier.
     static_assert(BK == 16, "the pipeline below is written for two groups of four k-steps per slab");
-    constexpr int NMFMA = 4 * TM * TN;  // MFMAs per group
-    const int a_col = wm * WM + (lane & 31), b_col = wn * WN + (lane & 31), khalf = lane >> 5;
-    float a0[TM][4], b0[TN][4], a1[TM][4], b1[TN][4];
-    // The body is unconditional so that each half of the loop is one scheduling region: past the
-    // end of K the write goes to a buffer nobody reads again and the fetch re-reads the last slab
-    // (unguarded path) or returns zeros (guarded path).  The slab count is rounded up to even; the
-    // unguarded path therefore requires K % 32 == 0, the guarded one multiplies a slab of zeros.
+    constexpr int ITEMS3 = 2 * NWR + NRB;
+    constexpr int IPS3 = (ITEMS3 + NMFMA - 2) / (NMFMA - 1);  // items behind each MFMA of S3, last one free
+    constexpr int IPS5 = (NRB + NMFMA - 2) / (NMFMA - 1);
+    // The body is unconditional: past the end of K the write goes to a buffer nobody reads again
+    // and the fetch re-reads the last slab (unguarded path) or returns zeros (guarded path).  The
+    // slab count is rounded up to even; the unguarded path therefore requires K % 32 == 0, the
+    // guarded one multiplies a slab of zeros.
     const int nk = ((p.K + BK - 1) / BK + 1) & ~1;
     const int k_last = GUARD ? (nk + 2) * BK : (nk - 1) * BK;
 #define SG_SLAB_BODY(KT, RA, RB)                                                               \
     do {                                                                                       \
         const int cur = (KT) & 1;                                                              \
-        SG_FETCH(lds_a[cur], lds_b[cur], 1, a1, b1);                                           \
-        TA::store(RA, lds_a[cur ^ 1], tid);                                                    \
-        TB::store(RB, lds_b[cur ^ 1], tid);                                                    \
-        SG_LOAD_SLAB(RA, RB, min(((KT) + 3) * BK, k_last));                                    \
-        SG_MFMA_GROUP(a0, b0);                                                                 \
-        _Pragma("unroll") for (int q = 0; q < NMFMA - 3; ++q) {                                \
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                 \
+        const int k_next = min(((KT) + 3) * BK, k_last);                                       \
+        _Pragma("unroll") for (int t = 0; t < NMFMA; ++t) {                                    \
+            SG_MFMA(t, a0, b0);                                                                \
+            __builtin_amdgcn_sched_barrier(0);                                                 \
+            _Pragma("unroll") for (int e = t * IPS3; e < (t + 1) * IPS3; ++e) {                \
+                if (e < NWR) SG_ITEM_STORE(e, RA, RB, cur ^ 1);                                \
+                else if (e < NWR + NRB) SG_ITEM_FETCH(e - NWR, cur, 1, a1, b1);                \
+                else if (e < ITEMS3) SG_ITEM_LOAD(e - NWR - NRB, RA, RB, k_next);              \
+            }                                                                                  \
+            __builtin_amdgcn_sched_barrier(0);                                                 \
         }                                                                                      \
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
-        __builtin_amdgcn_sched_group_barrier(0x200, TA::NV + TB::NV, 0);                       \
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
-        __builtin_amdgcn_sched_group_barrier(0x020, TA::NV + TB::NV, 0);                       \
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
         __syncthreads();                                                                       \
-        SG_FETCH(lds_a[cur ^ 1], lds_b[cur ^ 1], 0, a0, b0);                                   \
-        SG_MFMA_GROUP(a1, b1);                                                                 \
-        _Pragma("unroll") for (int q = 0; q < NMFMA; ++q) {                                    \
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);                                 \
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);                                 \
+        _Pragma("unroll") for (int t = 0; t < NMFMA; ++t) {                                    \
+            SG_MFMA(t, a1, b1);                                                                \
+            __builtin_amdgcn_sched_barrier(0);                                                 \
+            _Pragma("unroll") for (int e = t * IPS5; e < (t + 1) * IPS5; ++e) {                \
+                if (e < NRB) SG_ITEM_FETCH(e, cur ^ 1, 0, a0, b0);                             \
+            }                                                                                  \
+            __builtin_amdgcn_sched_barrier(0);                                                 \
         }                                                                                      \
     } while (0)
 
-    SG_LOAD_SLAB(ra0, rb0, 0);
-    SG_LOAD_SLAB(ra1, rb1, BK);
-    TA::store(ra0, lds_a[0], tid);
-    TB::store(rb0, lds_b[0], tid);
-    SG_LOAD_SLAB(ra0, rb0, min(2 * BK, k_last));
+#pragma unroll
+    for (int e = 0; e < NWR; ++e) SG_ITEM_LOAD(e, ra0, rb0, 0);
+#pragma unroll
+    for (int e = 0; e < NWR; ++e) SG_ITEM_LOAD(e, ra1, rb1, BK);
+#pragma unroll
+    for (int e = 0; e < NWR; ++e) SG_ITEM_STORE(e, ra0, rb0, 0);
+#pragma unroll
+    for (int e = 0; e < NWR; ++e) SG_ITEM_LOAD(e, ra0, rb0, min(2 * BK, k_last));
     __syncthreads();
-    SG_FETCH(lds_a[0], lds_b[0], 0, a0, b0);
+#pragma unroll
+    for (int e = 0; e < NRB; ++e) SG_ITEM_FETCH(e, 0, 0, a0, b0);
     for (int kt = 0; kt < nk; kt += 2) {
         SG_SLAB_BODY(kt, ra1, rb1);
         SG_SLAB_BODY(kt + 1, ra0, rb0);
     }
 #undef SG_SLAB_BODY
-#undef SG_LOAD_SLAB
-#undef SG_FETCH
-#undef SG_MFMA_GROUP
+#undef SG_ITEM_LOAD
+#undef SG_ITEM_STORE
+#undef SG_ITEM_FETCH
+#undef SG_MFMA
 
-    // ---- epilogue: element r of a 32x32 block sits at row (r/4)*8 + (lane/32)*4 + r%4, col lane%32
+    // ---- epilogue.  Element r of a 32x32 accumulator block sits at row (r/4)*8 + (lane/32)*4 + r%4,
+    // column lane%32.  Each wavefront passes its blocks one at a time through a private 32x32 LDS
+    // stage and reads them back as rows, so bias / residual / C move 16 bytes per lane in full
+    // 128-byte row segments.  Everything after the staging write is ONE rolled loop over the
+    // blocks: the kernel stays a few KB of code instead of an unrolled copy of the activation math
+    // per accumulator register, which costs microseconds of instruction fetch on every launch.
+    __syncthreads();  // all operand reads are done; the stage aliases the operand buffers
+    float *stage = lds_raw + wave * STAGE;
     float *C = p.C + bt0 * p.c_sb0 + bt1 * p.c_sb1;
     const float *R = p.res ? p.res + bt0 * p.r_sb0 + bt1 * p.r_sb1 : nullptr;
+    const int st_w = (khalf * 4) * STAGE_LD + (lane & 31);        // + ((r/4)*8 + r%4) * STAGE_LD
+    const int rd_row = lane >> 3, rd_col = (lane & 7) * 4;          // + 8q rows
+#pragma unroll 1
+    for (int blk = 0; blk < TM * TN; ++blk) {
+        // the accumulator block is chosen by a uniform branch so that register indices stay static
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int n = n0 + wn * WN + j * 32 + (lane & 31);
-        if (n >= p.N) continue;
-        const float bias = p.bias ? p.bias[n] : 0.0f;
+        for (int ij = 0; ij < TM * TN; ++ij) {
+            if (blk == ij) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm * WM + i * 32 + (r >> 2) * 8 + khalf * 4 + (r & 3);
-                if (m < p.M) {
-                    float v = acc[i][j][r];
-                    if (p.alpha != 1.0f) v *= p.alpha;
-                    if (p.bias) v += bias;
-                    v = apply_act(v, p.act);
-                    if (R) v += R[(int64_t)m * p.r_sm + n];
-                    v = apply_act(v, p.act_post);
-                    C[(int64_t)m * p.c_sm + n] = v;
-                }
+                for (int r = 0; r < 16; ++r) stage[st_w + ((r >> 2) * 8 + (r & 3)) * STAGE_LD] = acc[ij / TN][ij % TN][r];
             }
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int mb = m0 + wm * WM + (blk / TN) * 32, n = n0 + wn * WN + (blk % TN) * 32 + rd_col;
+        const bool n_in = !GUARD || n + 3 < p.N;
+        f32x4 bias = {0.f, 0.f, 0.f, 0.f};
+        if (p.bias) {
+            if (p.vec_bias && n_in) bias = *reinterpret_cast<const f32x4 *>(p.bias + n);
+            else {
+                if (n + 0 < p.N) bias.x = p.bias[n + 0];
+                if (n + 1 < p.N) bias.y = p.bias[n + 1];
+                if (n + 2 < p.N) bias.z = p.bias[n + 2];
+                if (n + 3 < p.N) bias.w = p.bias[n + 3];
+            }
+        }
+#pragma unroll 1
+        for (int q = 0; q < 4; ++q) {
+            const int row = q * 8 + rd_row, m = mb + row;
+            f32x4 v = *reinterpret_cast<const f32x4 *>(&stage[row * STAGE_LD + rd_col]);
+            if (GUARD && (m >= p.M || n >= p.N)) continue;
+            if (p.alpha != 1.0f) v *= p.alpha;
+            if (p.bias) v += bias;
+            if (p.act != SG_ACT_NONE) { v.x = apply_act(v.x, p.act); v.y = apply_act(v.y, p.act); v.z = apply_act(v.z, p.act); v.w = apply_act(v.w, p.act); }
+            if (R) {
+                const float *rp = R + (int64_t)m * p.r_sm + n;
+                if (p.vec_r && n_in) v += *reinterpret_cast<const f32x4 *>(rp);
+                else {
+                    v.x += rp[0];
+                    if (n + 1 < p.N) v.y += rp[1];
+                    if (n + 2 < p.N) v.z += rp[2];
+                    if (n + 3 < p.N) v.w += rp[3];
+                }
+            }
+            if (p.act_post != SG_ACT_NONE) { v.x = apply_act(v.x, p.act_post); v.y = apply_act(v.y, p.act_post); v.z = apply_act(v.z, p.act_post); v.w = apply_act(v.w, p.act_post); }
+            float *cp = C + (int64_t)m * p.c_sm + n;
+            if (p.vec_c && n_in) *reinterpret_cast<f32x4 *>(cp) = v;
+            else {
+                cp[0] = v.x;
+                if (n + 1 < p.N) cp[1] = v.y;
+                if (n + 2 < p.N) cp[2] = v.z;
+                if (n + 3 < p.N) cp[3] = v.w;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
@@ -422,6 +492,7 @@ int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c,
     auto mult4 = [](int64_t v) { return v % 4 == 0; };
     p.vec_a = ptr_aligned16(a.ptr) && mult4(a_kc ? p.a_sm : p.a_sk) && mult4(a.sb0) && mult4(a.sb1);
     p.vec_b = ptr_aligned16(b.ptr) && mult4(b_nc ? p.b_sk : p.b_sn) && mult4(b.sb0) && mult4(b.sb1);
+    p.vec_c = c.s_col == 1 && ptr_aligned16(c.ptr) && mult4(p.c_sm) && mult4(c.sb0) && mult4(c.sb1);
     if (epi) {
         p.alpha = epi->alpha;
         p.act = epi->act; p.act_post = epi->act_post;
@@ -433,6 +504,7 @@ int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c,
             if (t->dtype != SG_FLOAT) return sg_fail(ctx, SG_ERR_DTYPE, "gemm: bias must be fp32");
             if (sg_numel(t) != N || !sg_is_dense(t)) return sg_fail(ctx, SG_ERR_SHAPE, "gemm: bias must be dense with N = %d elements", N);
             p.bias = (const float *)t->base + t->offset;
+            p.vec_bias = ptr_aligned16(p.bias);
         }
         if (epi->residual) {
             const sg_tensor *t = epi->residual;
@@ -455,6 +527,7 @@ int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c,
                 p.r_sb1 = 0;
             }
             if (r > 4) return sg_fail(ctx, SG_ERR_SHAPE, "gemm: residual rank above 4");
+            p.vec_r = (N == 1 || t->strides[r - 1] == 1) && ptr_aligned16(p.res) && mult4(p.r_sm) && mult4(p.r_sb0) && mult4(p.r_sb1);
         }
     }
     return launch_gemm(ctx, p, nb0 * nb1, a_kc, b_nc);

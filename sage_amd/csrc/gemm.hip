@@ -334,12 +334,46 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     // 128-byte row segments.  Everything after the staging write is ONE rolled loop over the
     // blocks: the kernel stays a few KB of code instead of an unrolled copy of the activation math
     // per accumulator register, which costs microseconds of instruction fetch on every launch.
-    __syncthreads();  // all operand reads are done; the stage aliases the operand buffers
+    // The bias and residual values of a block are requested one block ahead (the first ones before
+    // the barrier), so the rolled loop never waits a full memory round trip per row group; inside
+    // the loop the four row groups' residuals sit in a small shift register to keep indices static.
     float *stage = lds_raw + wave * STAGE;
     float *C = p.C + bt0 * p.c_sb0 + bt1 * p.c_sb1;
     const float *R = p.res ? p.res + bt0 * p.r_sb0 + bt1 * p.r_sb1 : nullptr;
     const int st_w = (khalf * 4) * STAGE_LD + (lane & 31);        // + ((r/4)*8 + r%4) * STAGE_LD
     const int rd_row = lane >> 3, rd_col = (lane & 7) * 4;          // + 8q rows
+    auto request = [&](int blk, f32x4(&res)[4], f32x4 &bias) {
+        const int mb = m0 + wm * WM + (blk / TN) * 32, n = n0 + wn * WN + (blk % TN) * 32 + rd_col;
+        const bool n_in = !GUARD || n + 3 < p.N;
+        bias = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (p.bias) {
+            if (p.vec_bias && n_in) bias = *reinterpret_cast<const f32x4 *>(p.bias + n);
+            else {
+                if (n + 0 < p.N) bias.x = p.bias[n + 0];
+                if (n + 1 < p.N) bias.y = p.bias[n + 1];
+                if (n + 2 < p.N) bias.z = p.bias[n + 2];
+                if (n + 3 < p.N) bias.w = p.bias[n + 3];
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            res[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+            const int m = mb + q * 8 + rd_row;
+            if (R && (!GUARD || (m < p.M && n < p.N))) {
+                const float *rp = R + (int64_t)m * p.r_sm + n;
+                if (p.vec_r && n_in) res[q] = *reinterpret_cast<const f32x4 *>(rp);
+                else {
+                    res[q].x = rp[0];
+                    if (n + 1 < p.N) res[q].y = rp[1];
+                    if (n + 2 < p.N) res[q].z = rp[2];
+                    if (n + 3 < p.N) res[q].w = rp[3];
+                }
+            }
+        }
+    };
+    f32x4 res_c[4], res_n[4], bias_c, bias_n;
+    request(0, res_c, bias_c);
+    __syncthreads();  // all operand reads are done; the stage aliases the operand buffers
 #pragma unroll 1
     for (int blk = 0; blk < TM * TN; ++blk) {
         // the accumulator block is chosen by a uniform branch so that register indices stay static
@@ -350,39 +384,23 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
                 for (int r = 0; r < 16; ++r) stage[st_w + ((r >> 2) * 8 + (r & 3)) * STAGE_LD] = acc[ij / TN][ij % TN][r];
             }
         }
+        if (TM * TN > 1) request(min(blk + 1, TM * TN - 1), res_n, bias_n);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         const int mb = m0 + wm * WM + (blk / TN) * 32, n = n0 + wn * WN + (blk % TN) * 32 + rd_col;
         const bool n_in = !GUARD || n + 3 < p.N;
-        f32x4 bias = {0.f, 0.f, 0.f, 0.f};
-        if (p.bias) {
-            if (p.vec_bias && n_in) bias = *reinterpret_cast<const f32x4 *>(p.bias + n);
-            else {
-                if (n + 0 < p.N) bias.x = p.bias[n + 0];
-                if (n + 1 < p.N) bias.y = p.bias[n + 1];
-                if (n + 2 < p.N) bias.z = p.bias[n + 2];
-                if (n + 3 < p.N) bias.w = p.bias[n + 3];
-            }
-        }
 #pragma unroll 1
         for (int q = 0; q < 4; ++q) {
             const int row = q * 8 + rd_row, m = mb + row;
             f32x4 v = *reinterpret_cast<const f32x4 *>(&stage[row * STAGE_LD + rd_col]);
+            const f32x4 res = res_c[0];
+            res_c[0] = res_c[1]; res_c[1] = res_c[2]; res_c[2] = res_c[3];
             if (GUARD && (m >= p.M || n >= p.N)) continue;
             if (p.alpha != 1.0f) v *= p.alpha;
-            if (p.bias) v += bias;
+            if (p.bias) v += bias_c;
             if (p.act != SG_ACT_NONE) { v.x = apply_act(v.x, p.act); v.y = apply_act(v.y, p.act); v.z = apply_act(v.z, p.act); v.w = apply_act(v.w, p.act); }
-            if (R) {
-                const float *rp = R + (int64_t)m * p.r_sm + n;
-                if (p.vec_r && n_in) v += *reinterpret_cast<const f32x4 *>(rp);
-                else {
-                    v.x += rp[0];
-                    if (n + 1 < p.N) v.y += rp[1];
-                    if (n + 2 < p.N) v.z += rp[2];
-                    if (n + 3 < p.N) v.w += rp[3];
-                }
-            }
+            if (R) v += res;
             if (p.act_post != SG_ACT_NONE) { v.x = apply_act(v.x, p.act_post); v.y = apply_act(v.y, p.act_post); v.z = apply_act(v.z, p.act_post); v.w = apply_act(v.w, p.act_post); }
             float *cp = C + (int64_t)m * p.c_sm + n;
             if (p.vec_c && n_in) *reinterpret_cast<f32x4 *>(cp) = v;
@@ -392,6 +410,11 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
                 if (n + 2 < p.N) cp[2] = v.z;
                 if (n + 3 < p.N) cp[3] = v.w;
             }
+        }
+        if (TM * TN > 1) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) res_c[q] = res_n[q];
+            bias_c = bias_n;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();

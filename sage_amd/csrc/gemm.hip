@@ -54,6 +54,8 @@ struct GemmP {
     int act, act_post;
     int vec_a, vec_b;  // 16-byte loads are legal for this operand
     int vec_c, vec_r, vec_bias;  // 16-byte accesses are legal for C rows / residual rows / the bias
+    int k_chunk;      // split-K: workgroup z multiplies k in [z*k_chunk, min(K, (z+1)*k_chunk)); 0 = all of K
+    int64_t c_sz;     // split-K: element stride between the partial results of consecutive z
 };
 
 __device__ __forceinline__ float apply_act(float v, int act) {
@@ -193,8 +195,11 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     const int bt0 = blockIdx.y / p.nb1, bt1 = blockIdx.y % p.nb1;
-    const float *A = p.A + bt0 * p.a_sb0 + bt1 * p.a_sb1;
-    const float *B = p.B + bt0 * p.b_sb0 + bt1 * p.b_sb1;
+    // split-K: this workgroup's share of the k range, addressed from 0 through shifted bases
+    const int k_begin = p.k_chunk ? (int)blockIdx.z * p.k_chunk : 0;
+    const int Kloc = p.k_chunk ? min(p.K - k_begin, p.k_chunk) : p.K;
+    const float *A = p.A + bt0 * p.a_sb0 + bt1 * p.a_sb1 + (int64_t)k_begin * p.a_sk;
+    const float *B = p.B + bt0 * p.b_sb0 + bt1 * p.b_sb1 + (int64_t)k_begin * p.b_sk;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -220,11 +225,11 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     do {                                                                                       \
         if ((e) < TA::NV) {                                                                    \
             const int ia = (e) < TA::NV ? (e) : 0;                                         \
-            if (GUARD) TA::load_one_guarded(RA[ia], ia, A, m0, (k0), p.M, p.K, p.a_sm, p.a_sk, p.vec_a, tid); \
+            if (GUARD) TA::load_one_guarded(RA[ia], ia, A, m0, (k0), p.M, Kloc, p.a_sm, p.a_sk, p.vec_a, tid); \
             else TA::load_one_fast(RA[ia], ia, A, m0, (k0), p.a_sm, p.a_sk, tid);             \
         } else {                                                                               \
             const int ib = (e) >= TA::NV ? (e) - TA::NV : 0;                               \
-            if (GUARD) TB::load_one_guarded(RB[ib], ib, B, n0, (k0), p.N, p.K, p.b_sn, p.b_sk, p.vec_b, tid); \
+            if (GUARD) TB::load_one_guarded(RB[ib], ib, B, n0, (k0), p.N, Kloc, p.b_sn, p.b_sk, p.vec_b, tid); \
             else TB::load_one_fast(RB[ib], ib, B, n0, (k0), p.b_sn, p.b_sk, tid);             \
         }                                                                                      \
     } while (0)
@@ -280,7 +285,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     // and the fetch re-reads the last slab (unguarded path) or returns zeros (guarded path).  The
     // slab count is rounded up to even; the unguarded path therefore requires K % 32 == 0, the
     // guarded one multiplies a slab of zeros.
-    const int nk = ((p.K + BK - 1) / BK + 1) & ~1;
+    const int nk = ((Kloc + BK - 1) / BK + 1) & ~1;
     const int k_last = GUARD ? (nk + 2) * BK : (nk - 1) * BK;
 #define SG_SLAB_BODY(KT, RA, RB)                                                               \
     do {                                                                                       \
@@ -338,7 +343,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     // the barrier), so the rolled loop never waits a full memory round trip per row group; inside
     // the loop the four row groups' residuals sit in a small shift register to keep indices static.
     float *stage = lds_raw + wave * STAGE;
-    float *C = p.C + bt0 * p.c_sb0 + bt1 * p.c_sb1;
+    float *C = p.C + bt0 * p.c_sb0 + bt1 * p.c_sb1 + (int64_t)blockIdx.z * p.c_sz;
     const float *R = p.res ? p.res + bt0 * p.r_sb0 + bt1 * p.r_sb1 : nullptr;
     const int st_w = (khalf * 4) * STAGE_LD + (lane & 31);        // + ((r/4)*8 + r%4) * STAGE_LD
     const int rd_row = lane >> 3, rd_col = (lane & 7) * 4;          // + 8q rows
@@ -421,6 +426,51 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     }
 }
 
+// Split-K second pass: sums the partial products of the k ranges in ascending order (so the result
+// does not depend on scheduling) and applies the epilogue.  ws holds [split][batch][M][N] dense.
+template <bool VEC>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *__restrict__ ws, int nsplit, int64_t slice, const GemmP p,
+                                                            int64_t total) {
+    constexpr int W = VEC ? 4 : 1;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int ncol = p.N / W;
+    const int n = (int)(idx % ncol) * W;
+    const int64_t row = idx / ncol;
+    const int m = (int)(row % p.M);
+    const int bt = (int)(row / p.M), bt0 = bt / p.nb1, bt1 = bt % p.nb1;
+    const float *src = ws + row * p.N + n;
+    float v[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) v[i] = 0.0f;
+    for (int z = 0; z < nsplit; ++z) {
+        if (VEC) {
+            const f32x4 t = *reinterpret_cast<const f32x4 *>(src + z * slice);
+#pragma unroll
+            for (int i = 0; i < W; ++i) v[i] += t[i];
+        } else {
+            v[0] += src[z * slice];
+        }
+    }
+    const float *R = p.res ? p.res + bt0 * p.r_sb0 + bt1 * p.r_sb1 + (int64_t)m * p.r_sm + n : nullptr;
+    float *C = p.C + bt0 * p.c_sb0 + bt1 * p.c_sb1 + (int64_t)m * p.c_sm + n;
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+        float x = v[i];
+        if (p.alpha != 1.0f) x *= p.alpha;
+        if (p.bias) x += p.bias[n + i];
+        x = apply_act(x, p.act);
+        if (R) x += R[i];
+        x = apply_act(x, p.act_post);
+        v[i] = x;
+    }
+    if (VEC && p.vec_c) *reinterpret_cast<f32x4 *>(C) = f32x4{v[0], v[W > 1 ? 1 : 0], v[W > 2 ? 2 : 0], v[W > 3 ? 3 : 0]};
+    else {
+#pragma unroll
+        for (int i = 0; i < W; ++i) C[i] = v[i];
+    }
+}
+
 template <int BM, int BN, int WAVES_M, bool GUARD>
 void launch_layouts(sg_ctx *ctx, const GemmP &p, dim3 grid, bool a_kc, bool b_nc) {
     dim3 block(NTHREADS);
@@ -435,10 +485,60 @@ bool needs_guard(const GemmP &p, int bm, int bn) {
     return p.M % bm != 0 || p.N % bn != 0 || p.K % (2 * BK) != 0 || !p.vec_a || !p.vec_b;
 }
 
+// How many k ranges to split into.  Splitting pays when the output has too few tiles to occupy the
+// chip and K is long: each range becomes its own workgroup (grid z) writing a partial product, and a
+// second kernel sums them.  Ranges are multiples of 32 so that the unguarded loop stays legal.
+int choose_split(int num_cus, int64_t wgs, int K, int *k_chunk) {
+    const int64_t cus = num_cus > 0 ? num_cus : 256;
+    *k_chunk = 0;
+    const char *force = getenv("SAGE_GEMM_SPLITK");
+    int want;
+    if (force) want = atoi(force);
+    else {
+        if (wgs * 2 > cus || K < 512) return 1;
+        want = (int)((2 * cus + wgs - 1) / wgs);
+        if (want > K / 128) want = K / 128;
+        if (want > 32) want = 32;
+    }
+    if (want < 2) return 1;
+    int chunk = ((K + want - 1) / want + 31) / 32 * 32;
+    const int nsplit = (K + chunk - 1) / chunk;
+    if (nsplit < 2) return 1;
+    *k_chunk = chunk;
+    return nsplit;
+}
+
 template <int BM, int BN, int WAVES_M>
 int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
+    int k_chunk = 0;
+    const int nsplit = choose_split(ctx->num_cus, (int64_t)p.tiles_m * p.tiles_n * batch, p.K, &k_chunk);
+    if (nsplit > 1) {
+        const int64_t slice = (int64_t)batch * p.M * p.N;
+        void *ws = nullptr;
+        if (sg_alloc(ctx, (uint64_t)nsplit * slice * sizeof(float), &ws) == SG_OK) {
+            GemmP q = p;  // first pass: raw partial products into the workspace
+            q.C = (float *)ws;
+            q.c_sm = p.N; q.c_sb1 = (int64_t)p.M * p.N; q.c_sb0 = q.c_sb1 * p.nb1; q.c_sz = slice;
+            q.k_chunk = k_chunk;
+            q.bias = nullptr; q.res = nullptr; q.alpha = 1.0f; q.act = SG_ACT_NONE; q.act_post = SG_ACT_NONE;
+            q.vec_c = p.N % 4 == 0;
+            dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, (unsigned)nsplit);
+            if (needs_guard(p, BM, BN)) launch_layouts<BM, BN, WAVES_M, true>(ctx, q, grid, a_kc, b_nc);
+            else launch_layouts<BM, BN, WAVES_M, false>(ctx, q, grid, a_kc, b_nc);
+            SG_CHECK_LAUNCH(ctx, "gemm (split-K pass 1)");
+            const bool vec = p.N % 4 == 0;
+            const int64_t total = slice / (vec ? 4 : 1);
+            dim3 rgrid((unsigned)((total + 255) / 256));
+            if (vec) hipLaunchKernelGGL((splitk_reduce_kernel<true>), rgrid, dim3(256), 0, ctx->stream, (const float *)ws, nsplit, slice, p, total);
+            else hipLaunchKernelGGL((splitk_reduce_kernel<false>), rgrid, dim3(256), 0, ctx->stream, (const float *)ws, nsplit, slice, p, total);
+            SG_CHECK_LAUNCH(ctx, "gemm (split-K pass 2)");
+            // the block returns to the context's cache; later users are ordered behind these kernels on the stream
+            return sg_free(ctx, ws);
+        }
+        // no room for the workspace: fall through to the single-pass kernel
+    }
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
     if (needs_guard(p, BM, BN)) launch_layouts<BM, BN, WAVES_M, true>(ctx, p, grid, a_kc, b_nc);
     else launch_layouts<BM, BN, WAVES_M, false>(ctx, p, grid, a_kc, b_nc);

@@ -332,6 +332,46 @@ def test_gemm_modes(ctx, mkn, ta, tb):
     close(y, ref64, REL_GEMM, "gemm vs float64")
 
 
+@pytest.mark.parametrize("mkn,split", [((128, 4608, 512), None), ((512, 2304, 256), None), ((64, 1024, 64), None),
+                                       ((70, 999, 33), "5"), ((130, 257, 70), "3"), ((128, 512, 128), "32"), ((37, 2000, 41), "7")])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
+def test_gemm_split_k(ctx, monkeypatch, mkn, split, ta, tb):
+    """Few output tiles and a long K: the k range is split over workgroups and summed by a second kernel
+    (chosen by itself for the first three shapes, forced for the ragged ones), with the epilogue behind it."""
+    m, k, n = mkn
+    say("gemm split-K", mkn, split, ta, tb)
+    if split:
+        monkeypatch.setenv("SAGE_GEMM_SPLITK", split)
+    rng = np.random.default_rng(m + k + n)
+    a = rng.uniform(-1, 1, (k, m) if ta else (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (n, k) if tb else (k, n)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (n,)).astype(np.float32)
+    res = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    n0 = ctx.launches
+    y = nn.relu(V.gemm(dev(ctx, a), dev(ctx, b), ta, tb) + dev(ctx, bias)).eval(ctx).numpy()
+    assert ctx.launches - n0 == 1
+    ref64 = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+    close(y, np.maximum(ref64 + bias, 0), REL_GEMM, "relu(gemm + bias) vs float64")
+    close(y, O.relu(O.binary("add", O.gemm(ht(a), ht(b), ta, tb), ht(bias).expand([m, n]))).numpy(), REL_GEMM, "vs oracle")
+    y2 = ((V.gemm(dev(ctx, a), dev(ctx, b), ta, tb) + dev(ctx, bias)) + dev(ctx, res)).eval(ctx).numpy()
+    close(y2, ref64 + bias + res, REL_GEMM, "gemm + bias + residual vs float64")
+    # the split is summed in a fixed order: the same call gives the same bits
+    y3 = ((V.gemm(dev(ctx, a), dev(ctx, b), ta, tb) + dev(ctx, bias)) + dev(ctx, res)).eval(ctx).numpy()
+    exact(y2, y3, "run-to-run")
+
+
+def test_gemm_batched_split_k(ctx, monkeypatch):
+    say("gemm_batched split-K")
+    monkeypatch.setenv("SAGE_GEMM_SPLITK", "4")
+    rng = np.random.default_rng(77)
+    bt, m, k, n = 3, 37, 300, 44
+    a = rng.uniform(-1, 1, (bt, m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (bt, k, n)).astype(np.float32)
+    y = V.gemm_batched(dev(ctx, a), dev(ctx, b), False, False).eval(ctx).numpy()
+    close(y, np.einsum("bmk,bkn->bmn", a.astype(np.float64), b.astype(np.float64)), REL_GEMM, "batched split")
+    close(y, O.gemm_batched(ht(a), ht(b), False, False).numpy(), REL_GEMM, "vs oracle")
+
+
 def test_gemm_offsets_and_ld(ctx):
     """ld = strides[0] and element offsets, as gemm.rs:208-217 passes them: slices of larger matrices."""
     say("gemm ld/offset")

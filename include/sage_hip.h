@@ -254,6 +254,20 @@ int sg_softmax_cross_entropy(sg_ctx *ctx, const sg_tensor *logits, const sg_tens
 int sg_layer_norm_lastaxis(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *gamma,
                            const sg_tensor *beta, float eps, const sg_tensor *out);
 
+/* ---- fused attention: the operator chain of MultiHeadAttention::pass (bert.rs:262-271) --------- */
+
+/* out = softmax_lastaxis(scale * (q . k^T) + addend) . v, i.e. matmul_batched (gemm.rs:53-104), the
+ * division by sqrt(head size) and the mask addition (bert.rs:264-268), Softmax::pass on axis 3
+ * (layers.rs:266-273, nn.rs:42-56) and the second matmul_batched, without materialising the
+ * [Lq,Lk] scores.  q, out: [.., Lq, D]; k, v: [.., Lk, D]; rank 2..4, leading axes are batch axes
+ * with arbitrary strides (so the separate_heads views of bert.rs:282-291 and the merged-heads
+ * output layout of bert.rs:293-302 need no copies); unit stride on D; D = 32 or 64.
+ * addend: NULL or [.., Lq, Lk] holding one value per key (stride 0 over Lq, stride 1 over Lk, batch
+ * strides may be 0): the extended mask of bert.rs:304-314.  The softmax shift is max(0, row max)
+ * as in the reference (reduce.rs:282), so a fully masked row gives the reference's 0/0. */
+int sg_attention(sg_ctx *ctx, const sg_tensor *q, const sg_tensor *k, const sg_tensor *v,
+                 const sg_tensor *addend, float scale, const sg_tensor *out);
+
 #ifdef __cplusplus
 }
 #endif

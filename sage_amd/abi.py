@@ -88,6 +88,7 @@ PROTOTYPES = {
     "sg_softmax_lastaxis": (C.c_int, [_CTX, _TP, _TP, _TP]),
     "sg_softmax_cross_entropy": (C.c_int, [_CTX, _TP, _TP, _TP]),
     "sg_layer_norm_lastaxis": (C.c_int, [_CTX, _TP, _TP, _TP, C.c_float, _TP]),
+    "sg_attention": (C.c_int, [_CTX, _TP, _TP, _TP, _TP, C.c_float, _TP]),
 }
 
 _lib = None

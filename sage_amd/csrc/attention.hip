@@ -1,0 +1,289 @@
+// Scaled-dot-product attention in one kernel, fp32 on the CDNA4 matrix cores, for gfx950.
+//
+// Replaces the operator chain of MultiHeadAttention::pass (bert.rs:262-271):
+//   matmul_batched(q, k^T) -> div(sqrt(d)) -> add(extended mask) -> Softmax::pass(axis 3)
+//   -> matmul_batched(., v) -> merge_heads copy
+// i.e. two batched GEMMs (gemm.rs:53-104), two maps, the softmax composition of nn.rs:42-56 and an
+// organize() copy, none of which keeps the [L,L] scores out of memory.
+//
+// Design:
+//   * A workgroup of 4 wavefronts owns 128 queries of one (batch, head); a wavefront owns 32 of
+//     them for the whole kernel.  Keys and values are walked in blocks of 64 through LDS.
+//   * The score block is computed TRANSPOSED, S^T = K . Q^T (rows = keys, columns = queries), with
+//     v_mfma_f32_32x32x2_f32.  In the accumulator layout a lane then holds one query (lane % 32)
+//     and, in its 16 registers per 32-key block, the keys 8g + 4*(lane/32) + s (r = 4g + s).  That
+//     is exactly the k assignment the next product needs for its B operand, so the probabilities
+//     feed O^T = V^T . P^T straight from registers: no LDS round trip, no transposition.
+//   * Softmax is online over key blocks (running shift m and sum l per query).  A query lives in two
+//     lanes (l, l + 32), so the row statistics cost one cross-lane exchange.  The running shift
+//     starts at 0 and only grows: the result uses the shift max(0, row max), as the reference's
+//     softmax does (its max accumulator starts at literal 0, reduce.rs:282), including the 0/0 of a
+//     fully masked row.
+//   * O^T keeps the query in the lane as well, so rescaling by exp(m_old - m_new) and the final 1/l
+//     are per-lane scalars, and the output leaves as 16-byte pieces of a query's row.
+// Rounding differs from the reference's two-pass softmax and sequential-k products only at fp32
+// rounding level (covered by the 1e-3 tolerance of GEMM-bearing paths).
+#include "common.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int NW = 4;          // wavefronts per workgroup
+constexpr int QB = 32 * NW;    // queries per workgroup
+constexpr int KB = 64;         // keys per LDS block
+constexpr int NKB = KB / 32;   // 32-key MFMA blocks per LDS block
+
+struct AttnP {
+    const float *q, *k, *v, *add;
+    float *o;
+    int Lq, Lk, nb1;
+    int64_t q_sb0, q_sb1, q_sl, k_sb0, k_sb1, k_sl, v_sb0, v_sb1, v_sl, o_sb0, o_sb1, o_sl;
+    int64_t a_sb0, a_sb1;  // addend strides over the two batch axes (0 = broadcast); per key, stride 1
+    float scale;
+    int vec_q, vec_k, vec_v, vec_o;
+};
+
+template <int D>
+__global__ void __launch_bounds__(64 * NW) attention_kernel(const AttnP p) {
+    static_assert(D % 32 == 0 && D <= 64, "head size 32 or 64");
+    constexpr int LD = D + 4;              // LDS row stride (floats): 8 consecutive rows cover all banks
+    constexpr int ND = D / 32;             // 32-wide blocks of the head dimension
+    constexpr int NG = D / 8;              // groups of four k-steps over the head dimension
+    constexpr int ROWV = D / 4;            // 16-byte pieces per K/V row
+    constexpr int NLD = KB * ROWV / (64 * NW);  // 16-byte pieces of a K (or V) block per thread
+    __shared__ __attribute__((aligned(16))) float lds_k[KB * LD];
+    __shared__ __attribute__((aligned(16))) float lds_v[KB * LD];
+    __shared__ __attribute__((aligned(16))) float lds_m[KB];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int ql = lane & 31, h = lane >> 5;
+    const int bt0 = blockIdx.y / p.nb1, bt1 = blockIdx.y % p.nb1;
+    const int q0 = blockIdx.x * QB + wave * 32;
+    const float *Q = p.q + bt0 * p.q_sb0 + bt1 * p.q_sb1;
+    const float *K = p.k + bt0 * p.k_sb0 + bt1 * p.k_sb1;
+    const float *V = p.v + bt0 * p.v_sb0 + bt1 * p.v_sb1;
+    const float *A = p.add ? p.add + bt0 * p.a_sb0 + bt1 * p.a_sb1 : nullptr;
+
+    // Q^T operand of this lane: Q[q][8g + 4h + s] for g < NG, s < 4, pre-multiplied by nothing
+    float qreg[NG][4];
+    {
+        const int q = q0 + ql;
+        const float *row = Q + (int64_t)q * p.q_sl;
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            f32x4 t = {0.f, 0.f, 0.f, 0.f};
+            if (q < p.Lq) {
+                if (p.vec_q) t = *reinterpret_cast<const f32x4 *>(row + 8 * g + 4 * h);
+                else { t.x = row[8 * g + 4 * h]; t.y = row[8 * g + 4 * h + 1]; t.z = row[8 * g + 4 * h + 2]; t.w = row[8 * g + 4 * h + 3]; }
+            }
+            qreg[g][0] = t.x; qreg[g][1] = t.y; qreg[g][2] = t.z; qreg[g][3] = t.w;
+        }
+    }
+
+    floatx16 oacc[ND];
+#pragma unroll
+    for (int j = 0; j < ND; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[j][r] = 0.0f;
+    float m_run = 0.0f, l_run = 0.0f;  // shift (starts at the reference's 0) and this lane's share of the sum
+
+    // global -> registers for one K/V block; piece f of the block: row f / ROWV, floats 4*(f % ROWV)..
+    f32x4 kreg[NLD], vreg[NLD];
+    float mreg = 0.0f;
+    auto request = [&](int kb0) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int f = tid + i * 64 * NW;
+            const int row = f / ROWV, c = (f % ROWV) * 4;
+            const int key = kb0 + row;
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
+            if (key < p.Lk) {
+                const float *kp = K + (int64_t)key * p.k_sl + c, *vp = V + (int64_t)key * p.v_sl + c;
+                if (p.vec_k) a = *reinterpret_cast<const f32x4 *>(kp);
+                else { a.x = kp[0]; a.y = kp[1]; a.z = kp[2]; a.w = kp[3]; }
+                if (p.vec_v) b = *reinterpret_cast<const f32x4 *>(vp);
+                else { b.x = vp[0]; b.y = vp[1]; b.z = vp[2]; b.w = vp[3]; }
+            }
+            kreg[i] = a;
+            vreg[i] = b;
+        }
+        if (tid < KB) {
+            const int key = kb0 + tid;
+            mreg = key < p.Lk ? (A ? A[key] : 0.0f) : -__builtin_inff();  // keys past the end never count
+        }
+    };
+    auto deposit = [&]() {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int f = tid + i * 64 * NW;
+            const int row = f / ROWV, c = (f % ROWV) * 4;
+            *reinterpret_cast<f32x4 *>(&lds_k[row * LD + c]) = kreg[i];
+            *reinterpret_cast<f32x4 *>(&lds_v[row * LD + c]) = vreg[i];
+        }
+        if (tid < KB) lds_m[tid] = mreg;
+    };
+
+    request(0);
+    for (int kb0 = 0; kb0 < p.Lk; kb0 += KB) {
+        __syncthreads();  // everyone is done reading the previous block
+        deposit();
+        __syncthreads();
+        if (kb0 + KB < p.Lk) request(kb0 + KB);  // in flight during this block's arithmetic
+
+        // ---- S^T block: keys x queries, contraction over the head dimension
+        floatx16 sacc[NKB];
+#pragma unroll
+        for (int b = 0; b < NKB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[b][r] = 0.0f;
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            f32x4 a[NKB];
+#pragma unroll
+            for (int b = 0; b < NKB; ++b) a[b] = *reinterpret_cast<const f32x4 *>(&lds_k[(b * 32 + ql) * LD + 8 * g + 4 * h]);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int b = 0; b < NKB; ++b) sacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[b][s], qreg[g][s], sacc[b], 0, 0, 0);
+        }
+
+        // ---- scale, mask, online softmax.  Register r = 4g + s of block b is key 32b + 8g + 4h + s.
+        float mloc = -__builtin_inff();
+#pragma unroll
+        for (int b = 0; b < NKB; ++b)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 mk = *reinterpret_cast<const f32x4 *>(&lds_m[b * 32 + 8 * g + 4 * h]);
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const float x = sacc[b][4 * g + s] * p.scale + mk[s];
+                    sacc[b][4 * g + s] = x;
+                    mloc = fmaxf(mloc, x);
+                }
+            }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+        const float m_new = fmaxf(m_run, mloc);
+        const float corr = expf(m_run - m_new);
+        m_run = m_new;
+        float lsum = 0.0f;
+#pragma unroll
+        for (int b = 0; b < NKB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float e = expf(sacc[b][r] - m_new);
+                sacc[b][r] = e;
+                lsum += e;
+            }
+        l_run = l_run * corr + lsum;
+#pragma unroll
+        for (int j = 0; j < ND; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[j][r] *= corr;
+
+        // ---- O^T += V^T . P^T: rows = head dimension, columns = queries, contraction over keys
+#pragma unroll
+        for (int b = 0; b < NKB; ++b)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float a[ND][4];
+#pragma unroll
+                for (int j = 0; j < ND; ++j)
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) a[j][s] = lds_v[(b * 32 + 8 * g + 4 * h + s) * LD + j * 32 + ql];
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+#pragma unroll
+                    for (int j = 0; j < ND; ++j) oacc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][s], sacc[b][4 * g + s], oacc[j], 0, 0, 0);
+            }
+    }
+
+    // ---- normalise and write: register r = 4g + s of block j is head index 32j + 8g + 4h + s
+    const float l = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = 1.0f / l;
+    const int q = q0 + ql;
+    if (q < p.Lq) {
+        float *row = p.o + bt0 * p.o_sb0 + bt1 * p.o_sb1 + (int64_t)q * p.o_sl;
+#pragma unroll
+        for (int j = 0; j < ND; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                f32x4 t = {oacc[j][4 * g] * inv, oacc[j][4 * g + 1] * inv, oacc[j][4 * g + 2] * inv, oacc[j][4 * g + 3] * inv};
+                float *dst = row + 32 * j + 8 * g + 4 * h;
+                if (p.vec_o) *reinterpret_cast<f32x4 *>(dst) = t;
+                else { dst[0] = t.x; dst[1] = t.y; dst[2] = t.z; dst[3] = t.w; }
+            }
+    }
+}
+
+bool aligned16(const void *base, int64_t offset_elems) { return ((uintptr_t)base + (uint64_t)offset_elems * 4) % 16 == 0; }
+
+// [.., L, D] operand with up to two leading batch axes -> (pointer, batch strides, row stride)
+int operand(sg_ctx *ctx, const sg_tensor *t, const char *who, int rank, const int64_t *batch, int64_t L, int64_t D, const float **ptr,
+            int64_t *sb0, int64_t *sb1, int64_t *sl, int *vec) {
+    int rc = sg_validate_tensor(ctx, t, who);
+    if (rc != SG_OK) return rc;
+    if (t->dtype != SG_FLOAT) return sg_fail(ctx, SG_ERR_DTYPE, "%s: fp32 only", who);
+    if (t->rank != rank) return sg_fail(ctx, SG_ERR_SHAPE, "%s: rank %d, expected %d", who, t->rank, rank);
+    for (int i = 0; i < rank - 2; ++i)
+        if (t->extents[i] != batch[i]) return sg_fail(ctx, SG_ERR_SHAPE, "%s: batch extents differ", who);
+    if (t->extents[rank - 2] != L || t->extents[rank - 1] != D) return sg_fail(ctx, SG_ERR_SHAPE, "%s: expected [.., %lld, %lld]", who, (long long)L, (long long)D);
+    if (t->strides[rank - 1] != 1) return sg_fail(ctx, SG_ERR_SHAPE, "%s: the head dimension must have unit stride", who);
+    *ptr = (const float *)t->base + t->offset;
+    *sl = t->strides[rank - 2];
+    *sb1 = rank >= 3 ? t->strides[rank - 3] : 0;
+    *sb0 = rank >= 4 ? t->strides[rank - 4] : 0;
+    *vec = aligned16(t->base, t->offset) && *sl % 4 == 0 && *sb0 % 4 == 0 && *sb1 % 4 == 0;
+    return SG_OK;
+}
+
+}  // namespace
+
+extern "C" int sg_attention(sg_ctx *ctx, const sg_tensor *q, const sg_tensor *k, const sg_tensor *v, const sg_tensor *addend, float scale,
+                            const sg_tensor *out) {
+    if (!ctx || !q || !k || !v || !out) return SG_ERR_ARG;
+    const int rank = q->rank;
+    if (rank < 2 || rank > 4) return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention: rank 2..4");
+    if (k->rank != rank) return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention: k rank differs");
+    const int64_t Lq = q->extents[rank - 2], D = q->extents[rank - 1], Lk = k->extents[rank - 2];
+    if (D != 32 && D != 64) return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention: head size %lld (32 and 64 are built)", (long long)D);
+    if (Lq < 1 || Lk < 1) return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention: empty sequence");
+    int64_t batch[2] = {1, 1};
+    for (int i = 0; i < rank - 2; ++i) batch[i] = q->extents[i];
+    AttnP p{};
+    int rc;
+    const float *optr;
+    if ((rc = operand(ctx, q, "sg_attention q", rank, batch, Lq, D, &p.q, &p.q_sb0, &p.q_sb1, &p.q_sl, &p.vec_q)) != SG_OK) return rc;
+    if ((rc = operand(ctx, k, "sg_attention k", rank, batch, Lk, D, &p.k, &p.k_sb0, &p.k_sb1, &p.k_sl, &p.vec_k)) != SG_OK) return rc;
+    if ((rc = operand(ctx, v, "sg_attention v", rank, batch, Lk, D, &p.v, &p.v_sb0, &p.v_sb1, &p.v_sl, &p.vec_v)) != SG_OK) return rc;
+    if ((rc = operand(ctx, out, "sg_attention out", rank, batch, Lq, D, &optr, &p.o_sb0, &p.o_sb1, &p.o_sl, &p.vec_o)) != SG_OK) return rc;
+    p.o = const_cast<float *>(optr);
+    int64_t nb0 = 1, nb1 = 1;
+    if (rank == 3) nb1 = batch[0];
+    if (rank == 4) { nb0 = batch[0]; nb1 = batch[1]; }
+    if (addend) {
+        if ((rc = sg_validate_tensor(ctx, addend, "sg_attention addend")) != SG_OK) return rc;
+        if (addend->dtype != SG_FLOAT) return sg_fail(ctx, SG_ERR_DTYPE, "sg_attention addend: fp32 only");
+        if (addend->rank != rank) return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention addend: rank differs");
+        for (int i = 0; i < rank - 2; ++i)
+            if (addend->extents[i] != batch[i]) return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention addend: batch extents differ (broadcast with stride 0)");
+        if (addend->extents[rank - 2] != Lq || addend->extents[rank - 1] != Lk) return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention addend: expected [.., Lq, Lk]");
+        if ((Lq > 1 && addend->strides[rank - 2] != 0) || (Lk > 1 && addend->strides[rank - 1] != 1))
+            return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention addend: one value per key (query stride 0, key stride 1)");
+        p.add = (const float *)addend->base + addend->offset;
+        p.a_sb1 = rank >= 3 ? addend->strides[rank - 3] : 0;
+        p.a_sb0 = rank >= 4 ? addend->strides[rank - 4] : 0;
+    }
+    if (rank == 3) {  // the single batch axis is b1
+        p.q_sb0 = p.k_sb0 = p.v_sb0 = p.o_sb0 = p.a_sb0 = 0;
+    }
+    p.Lq = (int)Lq; p.Lk = (int)Lk; p.nb1 = (int)nb1;
+    p.scale = scale;
+    if (nb0 * nb1 > 65535) return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention: more than 65535 (batch x head) pairs");
+    dim3 grid((unsigned)((Lq + QB - 1) / QB), (unsigned)(nb0 * nb1));
+    if (D == 64) hipLaunchKernelGGL((attention_kernel<64>), grid, dim3(64 * NW), 0, ctx->stream, p);
+    else hipLaunchKernelGGL((attention_kernel<32>), grid, dim3(64 * NW), 0, ctx->stream, p);
+    SG_CHECK_LAUNCH(ctx, "attention");
+    return SG_OK;
+}

@@ -19,6 +19,7 @@ covers, never in values:
 the parity tests compare the fused results against.
 """
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -890,7 +891,70 @@ class _Evaluator:
     def _ev_gemm(self, v):
         return self.run_gemm(v)
 
-    _ev_gemm_batched = _ev_matmul_nd = _ev_gemm
+    _ev_gemm_batched = _ev_gemm
+
+    def _ev_matmul_nd(self, v):
+        if _FUSION["on"]:
+            t = self.try_attention(v, None)
+            if t is not None:
+                return t
+        return self.run_gemm(v)
+
+    # ---- pattern: softmax(scale * q.k^T + per-key addend) . v  (bert.rs:262-271) as one kernel
+    def _private(self, v):
+        """v is consumed exactly once, not yet evaluated and not asked for by the caller."""
+        return not self.done(v) and self.n_users(v) == 1 and id(v) not in self.targets
+
+    def try_attention(self, g, dest):
+        pr, vv = g.inputs
+        if os.environ.get("SAGE_FUSE_ATTENTION", "1") == "0":  # measurement switch: run the chain operator by operator
+            return None
+        if g.op != "matmul_nd" or pr.op != "softmax" or not self._private(pr) or g.rank > 4:
+            return None
+        x = pr.inputs[0]
+        add = None
+        if x.op == "binary" and x.attrs["name"] == "add" and self._private(x):
+            cands = [(x.inputs[0], x.inputs[1]), (x.inputs[1], x.inputs[0])]
+        else:
+            cands = [(x, None)]
+        for s_node, add in cands:
+            chain = [x] if add is not None else []
+            scale = 1.0
+            inner = s_node
+            if (s_node.op == "binary" and s_node.attrs["name"] in ("mul", "div") and s_node.inputs[1].op == "literal"
+                    and s_node.inputs[1].dtype == FLOAT):
+                lit = float(np.float32(s_node.inputs[1].attrs["value"]))
+                if s_node.attrs["name"] == "div":
+                    if lit == 0.0 or np.frexp(lit)[0] != 0.5:  # x/c == x*(1/c) only for powers of two
+                        continue
+                    lit = 1.0 / lit
+                chain.append(s_node)
+                scale, inner = lit, s_node.inputs[0]
+            chain.append(inner)
+            if inner.op != "matmul_nd" or inner.rank != g.rank or not all(self._private(n) for n in chain):
+                continue
+            qv, ktv = inner.inputs
+            d = qv.extents[-1]
+            if d not in (32, 64) or vv.extents[-1] != d or qv.dtype != FLOAT or vv.dtype != FLOAT:
+                continue
+            q, kt, vt = self.get(qv), self.get(ktv), self.get(vv)
+            r = g.rank
+            k = kt.with_shape(kt.shape.swap(r - 2, r - 1))
+            if q.strides[-1] != 1 or k.strides[-1] != 1 or vt.strides[-1] != 1:
+                continue
+            at = None
+            if add is not None:
+                at = self.get(add)
+                if (at.rank != r or at.extents != inner.extents or at.dtype != FLOAT
+                        or (at.extents[-2] > 1 and at.strides[-2] != 0) or (at.extents[-1] > 1 and at.strides[-1] != 1)):
+                    continue
+            y = dest if dest is not None else self.out(g.extents, FLOAT)
+            qc, kc, vc, yc = q.c(), k.c(), vt.c(), y.c()
+            ac = at.c() if at is not None else None
+            self.call(self.lib.sg_attention, C.byref(qc), C.byref(kc), C.byref(vc), C.byref(ac) if ac is not None else None,
+                      C.c_float(scale), C.byref(yc))
+            return y
+        return None
 
     # ---- pattern: maps that directly consume a GEMM become its epilogue
     @staticmethod
@@ -1175,7 +1239,8 @@ class _Evaluator:
         for i, a in enumerate(axes):
             inv[a] = i
         dest = y.with_shape(y.shape.permute(inv))  # g's extents over y's memory
-        self.run_gemm(g, None, dest)
+        if self.try_attention(g, dest) is None:
+            self.run_gemm(g, None, dest)
         return y
 
     # ---- fused row operators

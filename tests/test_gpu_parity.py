@@ -4,6 +4,8 @@ Bar: indexing, gather, argmax, compare/logic results and pure +,-,*,/ arithmetic
 transcendental maps and reductions agree within rel 1e-4; GEMM, convolution and model outputs
 within rel 1e-3 (tests/util.py).  Every test prints its case before touching the GPU.
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -540,6 +542,85 @@ def test_softmax_with_mask_addend(ctx):
     close(dev_expr().eval(ctx).numpy(), yo, REL_MAP, "fused")
     V.set_fusion(False)
     close(dev_expr().eval(ctx).numpy(), yo, REL_MAP, "composed")
+
+
+def _attention_f64(q, k, v, mask_add, scale):
+    s = np.einsum("...qd,...kd->...qk", q.astype(np.float64), k.astype(np.float64)) * scale
+    if mask_add is not None:
+        s = s + mask_add
+    e = np.exp(s - np.maximum(s.max(-1, keepdims=True), 0.0))
+    return np.einsum("...qk,...kd->...qd", e / e.sum(-1, keepdims=True), v.astype(np.float64))
+
+
+@pytest.mark.parametrize("n,h,lq,lk,d", [(2, 3, 128, 128, 64), (1, 2, 70, 70, 64), (2, 2, 33, 200, 32), (1, 1, 1, 5, 64), (3, 12, 256, 256, 64)])
+@pytest.mark.parametrize("masked", [False, True])
+def test_attention_fused_vs_composed_vs_oracle(ctx, n, h, lq, lk, d, masked):
+    """softmax(q.k^T / sqrt(d) + mask) . v on the separate_heads views of bert.rs:282-291, merged back as
+    bert.rs:293-302: one launch when fused; equal to the operator-by-operator result and the oracle."""
+    say("attention", n, h, lq, lk, d, masked)
+    rng = np.random.default_rng(n * 1000 + lq + lk + d)
+    e = h * d
+    qa, ka, va = (rng.standard_normal((n, l_, e)).astype(np.float32) for l_ in (lq, lk, lk))
+    m = (rng.uniform(0, 1, (n, lk)) > 0.3).astype(np.float32)
+    m[:, 0] = 1.0
+    scale = float(np.sqrt(np.float32(d)))
+
+    def heads(f, l_):
+        return f.view([n, l_, h, d]).transpose(2, 1)
+
+    def expr(mk):
+        q, k, v = heads(mk(qa), lq), heads(mk(ka), lk), heads(mk(va), lk)
+        att = q.matmul_batched(k.transpose(-1, -2))
+        att = att / scale if d == 64 else att * (1.0 / scale)  # a division folds only when exact (power of two)
+        if masked:
+            att = att + (-mk(m).view([n, 1, 1, lk]) + 1.0) * -1e5
+        return att, v
+
+    att, v = expr(lambda a: dev(ctx, a))
+    n0 = ctx.launches
+    out = nn.softmax(att, 3).matmul_batched(v).transpose(2, 1)
+    yf = out.view([n, lq, e]).eval(ctx).numpy()
+    fused_launches = ctx.launches - n0
+    V.set_fusion(False)
+    att, v = expr(lambda a: dev(ctx, a))
+    yc = nn.softmax(att, 3).matmul_batched(v).transpose(2, 1).view([n, lq, e]).eval(ctx).numpy()
+    qh, kh, vh = (a.reshape(n, l_, h, d).transpose(0, 2, 1, 3) for a, l_ in ((qa, lq), (ka, lk), (va, lk)))
+    madd = ((1.0 - m.astype(np.float64)) * -1e5)[:, None, None, :] if masked else None
+    ref = _attention_f64(qh, kh, vh, madd, 1.0 / scale).transpose(0, 2, 1, 3).reshape(n, lq, e)
+    close(yf, ref, REL_GEMM, "fused vs float64")
+    close(yc, ref, REL_GEMM, "composed vs float64")
+    close(yf, yc, REL_GEMM, "fused vs composed")
+    assert fused_launches == (2 if masked else 1), fused_launches  # the mask expression + the attention kernel
+
+
+def test_attention_fully_masked_row_is_reference_nan(ctx):
+    """Every key masked by -1e5: the reference's softmax shifts by max(0, row max) = 0, every exp underflows
+    and the row is 0/0.  The fused kernel keeps that behaviour instead of a uniform row."""
+    say("attention fully masked")
+    rng = np.random.default_rng(5)
+    n, h, l, d = 2, 2, 64, 64
+    qa, ka, va = (rng.standard_normal((n, l, h * d)).astype(np.float32) for _ in range(3))
+    m = np.ones((n, l), np.float32)
+    m[1, :] = 0.0
+
+    def run():
+        hd = lambda a: dev(ctx, a).view([n, l, h, d]).transpose(2, 1)
+        att = hd(qa).matmul_batched(hd(ka).transpose(-1, -2)) / 8.0 + (-dev(ctx, m).view([n, 1, 1, l]) + 1.0) * -1e5
+        return nn.softmax(att, 3).matmul_batched(hd(va)).eval(ctx).numpy()
+
+    yf = run()
+    V.set_fusion(False)
+    yc = run()
+    assert np.isnan(yf[1]).all() and np.isnan(yc[1]).all()
+    close(yf[0], yc[0], REL_GEMM, "unmasked batch")
+
+
+def test_attention_abi_errors(ctx):
+    say("attention errors")
+    q = S.Tensor.uninit(ctx, [2, 16, 48])
+    with pytest.raises(abi.ShapeError):
+        qc = q.c()
+        ctx.check(ctx._lib.sg_attention(ctx.handle, C.byref(qc), C.byref(qc), C.byref(qc), None, C.c_float(1.0), C.byref(qc)))
 
 
 @pytest.mark.parametrize("shape", [(5, 10), (512, 1024), (37, 1000), (16, 4096)])

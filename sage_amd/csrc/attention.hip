@@ -165,14 +165,18 @@ __global__ void __launch_bounds__(64 * NW) attention_kernel(const AttnP p) {
             }
         mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
         const float m_new = fmaxf(m_run, mloc);
-        const float corr = expf(m_run - m_new);
+        // exp(x - m) as 2^(x*log2(e) - m*log2(e)): one fused multiply-add and the hardware exp2; the argument
+        // rounding costs about |x - m| * 6e-8 relative, far inside the softmax tolerance
+        constexpr float LOG2E = 1.44269504088896340736f;
+        const float corr = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
+        const float mshift = -m_new * LOG2E;
         m_run = m_new;
         float lsum = 0.0f;
 #pragma unroll
         for (int b = 0; b < NKB; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float e = expf(sacc[b][r] - m_new);
+                const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[b][r], LOG2E, mshift));
                 sacc[b][r] = e;
                 lsum += e;
             }

@@ -616,6 +616,34 @@ class Program:
         return self.outputs
 
 
+def _merge_common_subgraphs(targets):
+    """Structurally identical operations on the same inputs are computed once: inputs of every node are
+    re-pointed at the first node seen with the same (operator, attributes, inputs).  BERT rebuilds the
+    extended attention mask in each of its layers (bert.rs:264-268, 304-314); this leaves one."""
+    canon, table = {}, {}
+    order, seen, stack = [], set(), [(t, False) for t in targets]
+    while stack:
+        v, expanded = stack.pop()
+        if expanded:
+            order.append(v)
+            continue
+        if id(v) in seen:
+            continue
+        seen.add(id(v))
+        stack.append((v, True))
+        if v.value is None:
+            for i in v.inputs:
+                stack.append((i, False))
+    for v in order:
+        if v.value is not None or v.op == "data":
+            canon[id(v)] = v
+            continue
+        v.inputs = tuple(canon[id(i)] for i in v.inputs)
+        key = (v.op, v.dtype, tuple(v.shape.extents), tuple(v.shape.strides), v.shape.offset,
+               repr(sorted(v.attrs.items(), key=lambda kv: kv[0])), tuple(id(i) for i in v.inputs))
+        canon[id(v)] = table.setdefault(key, v)
+
+
 class _Evaluator:
     def __init__(self, ctx, targets, record=None):
         self.ctx = ctx
@@ -623,6 +651,8 @@ class _Evaluator:
         self.memo = {}
         self.users = {}
         self.targets = {id(t) for t in targets}
+        if _FUSION["on"]:
+            _merge_common_subgraphs(targets)
         seen = set()
         stack = list(targets)
         while stack:

@@ -268,6 +268,21 @@ int sg_layer_norm_lastaxis(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *gam
 int sg_attention(sg_ctx *ctx, const sg_tensor *q, const sg_tensor *k, const sg_tensor *v,
                  const sg_tensor *addend, float scale, const sg_tensor *out);
 
+/* ---- replay of a recorded launch sequence --------------------------------------------------- */
+
+/* Counterpart of replaying a compiled Program (Program::exec, session.rs:208-468) without the host
+ * loop: every launch issued on the context between sg_graph_begin and sg_graph_end is recorded into
+ * a HIP graph instead of being executed; sg_graph_launch replays all of them, on the same buffers,
+ * with one submission.  Calls that wait for the device (sg_memcpy_h2d, sg_memcpy_d2h, sg_sync) are
+ * refused inside a capture.  Workspaces the library allocates for captured kernels (split-K partial
+ * products) stay allocated until sg_graph_destroy.  The expression kernels of sg_map must have
+ * been built before the capture (run the sequence once first). */
+typedef struct sg_graph sg_graph;
+int sg_graph_begin(sg_ctx *ctx);
+int sg_graph_end(sg_ctx *ctx, sg_graph **out);
+int sg_graph_launch(sg_ctx *ctx, sg_graph *graph);
+int sg_graph_destroy(sg_ctx *ctx, sg_graph *graph);
+
 #ifdef __cplusplus
 }
 #endif

@@ -88,6 +88,10 @@ PROTOTYPES = {
     "sg_softmax_lastaxis": (C.c_int, [_CTX, _TP, _TP, _TP]),
     "sg_softmax_cross_entropy": (C.c_int, [_CTX, _TP, _TP, _TP]),
     "sg_layer_norm_lastaxis": (C.c_int, [_CTX, _TP, _TP, _TP, C.c_float, _TP]),
+    "sg_graph_begin": (C.c_int, [_CTX]),
+    "sg_graph_end": (C.c_int, [_CTX, C.POINTER(C.c_void_p)]),
+    "sg_graph_launch": (C.c_int, [_CTX, C.c_void_p]),
+    "sg_graph_destroy": (C.c_int, [_CTX, C.c_void_p]),
     "sg_attention": (C.c_int, [_CTX, _TP, _TP, _TP, _TP, C.c_float, _TP]),
 }
 

@@ -36,9 +36,19 @@ struct sg_ctx {
     std::multimap<uint64_t, void *> cache;
     // run-time built kernels keyed by their full source text (session/context.rs:62-83)
     std::unordered_map<std::string, sg_jit_kernel> jit;
+    // stream capture (sg_graph_begin .. sg_graph_end): blocks allocated AND freed inside the captured
+    // region are workspaces whose addresses are baked into the graph; they stay live with the graph
+    bool capturing = false;
+    std::vector<void *> capture_allocs, capture_held;
     // errors
     std::string last_error;
     uint64_t oom_needed = 0, oom_total = 0;
+};
+
+struct sg_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    std::vector<void *> held;  // workspaces the captured kernels use on every replay
 };
 
 int sg_fail(sg_ctx *ctx, int code, const char *fmt, ...);

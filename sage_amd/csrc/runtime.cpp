@@ -114,7 +114,7 @@ int sg_alloc(sg_ctx *ctx, uint64_t nbytes, void **dptr) {
         ctx->cache.erase(it);
     } else {
         hipError_t e = hipMalloc(&p, sz);
-        if (e != hipSuccess) {
+        if (e != hipSuccess && !ctx->capturing) {  // trimming synchronises, which a capture forbids
             (void)hipGetLastError();
             int rc = sg_trim(ctx);
             if (rc != SG_OK) return rc;
@@ -130,6 +130,7 @@ int sg_alloc(sg_ctx *ctx, uint64_t nbytes, void **dptr) {
         ctx->reserved += sz;
     }
     ctx->live[p] = sg_block{sz, nbytes};
+    if (ctx->capturing) ctx->capture_allocs.push_back(p);
     ctx->used += nbytes;
     if (ctx->used > ctx->peak) ctx->peak = ctx->used;
     *dptr = p;
@@ -141,6 +142,13 @@ int sg_free(sg_ctx *ctx, void *dptr) {
     if (!dptr) return SG_OK;
     auto it = ctx->live.find(dptr);
     if (it == ctx->live.end()) return sg_fail(ctx, SG_ERR_ARG, "sg_free: %p was not allocated by this context", dptr);
+    if (ctx->capturing) {
+        for (void *q : ctx->capture_allocs)
+            if (q == dptr) {  // a workspace of the captured kernels: it belongs to the graph from now on
+                ctx->capture_held.push_back(dptr);
+                return SG_OK;
+            }
+    }
     ctx->used -= it->second.requested;
     // Work already queued on the context's in-order stream finishes before any later launch that
     // is handed this block again, so the block can be reused without a device synchronisation.
@@ -161,6 +169,7 @@ int sg_mem_stats(sg_ctx *ctx, uint64_t *used, uint64_t *reserved, uint64_t *peak
 int sg_memcpy_h2d(sg_ctx *ctx, void *dst_dev, const void *src_host, uint64_t nbytes) {
     if (!ctx || (!dst_dev && nbytes) || (!src_host && nbytes)) return SG_ERR_ARG;
     if (!nbytes) return SG_OK;
+    if (ctx->capturing) return sg_fail(ctx, SG_ERR_ARG, "sg_memcpy_h2d waits for the stream and cannot be captured into a graph");
     SG_HIP(ctx, hipMemcpyAsync(dst_dev, src_host, nbytes, hipMemcpyHostToDevice, ctx->stream));
     SG_HIP(ctx, hipStreamSynchronize(ctx->stream));
     return SG_OK;
@@ -169,6 +178,7 @@ int sg_memcpy_h2d(sg_ctx *ctx, void *dst_dev, const void *src_host, uint64_t nby
 int sg_memcpy_d2h(sg_ctx *ctx, void *dst_host, const void *src_dev, uint64_t nbytes) {
     if (!ctx || (!dst_host && nbytes) || (!src_dev && nbytes)) return SG_ERR_ARG;
     if (!nbytes) return SG_OK;
+    if (ctx->capturing) return sg_fail(ctx, SG_ERR_ARG, "sg_memcpy_d2h waits for the stream and cannot be captured into a graph");
     SG_HIP(ctx, hipMemcpyAsync(dst_host, src_dev, nbytes, hipMemcpyDeviceToHost, ctx->stream));
     SG_HIP(ctx, hipStreamSynchronize(ctx->stream));
     return SG_OK;
@@ -183,6 +193,7 @@ int sg_memcpy_d2d(sg_ctx *ctx, void *dst_dev, const void *src_dev, uint64_t nbyt
 
 int sg_sync(sg_ctx *ctx) {
     if (!ctx) return SG_ERR_ARG;
+    if (ctx->capturing) return sg_fail(ctx, SG_ERR_ARG, "sg_sync waits for the stream and cannot be captured into a graph");
     SG_HIP(ctx, hipStreamSynchronize(ctx->stream));
     return SG_OK;
 }
@@ -228,3 +239,57 @@ int sg_last_oom(sg_ctx *ctx, uint64_t *needed, uint64_t *total) {
 int sg_kernel_cache_size(sg_ctx *ctx) { return ctx ? (int)ctx->jit.size() : -1; }
 
 }  // extern "C"
+
+// ---- HIP graphs: a recorded sequence of launches replayed with one submission ---------------------
+// The reference replays a compiled Program launch by launch (session.rs:208-468); a launch-bound
+// program (dozens of microsecond kernels) is bounded by that host loop.  Everything the library
+// launches goes to the context's stream, so a stream capture between begin and end records it.
+
+int sg_graph_begin(sg_ctx *ctx) {
+    if (!ctx) return SG_ERR_ARG;
+    if (ctx->capturing) return sg_fail(ctx, SG_ERR_ARG, "sg_graph_begin: a capture is already open");
+    SG_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+    ctx->capturing = true;
+    ctx->capture_allocs.clear();
+    ctx->capture_held.clear();
+    return SG_OK;
+}
+
+int sg_graph_end(sg_ctx *ctx, sg_graph **out) {
+    if (!ctx || !out) return SG_ERR_ARG;
+    *out = nullptr;
+    if (!ctx->capturing) return sg_fail(ctx, SG_ERR_ARG, "sg_graph_end: no capture is open");
+    ctx->capturing = false;
+    sg_graph *g = new sg_graph();
+    g->held.swap(ctx->capture_held);
+    ctx->capture_allocs.clear();
+    hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
+    if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        if (g->graph) (void)hipGraphDestroy(g->graph);
+        for (void *p : g->held) (void)sg_free(ctx, p);
+        delete g;
+        return sg_fail(ctx, SG_ERR_DEVICE, "graph capture failed: %s", hipGetErrorString(e));
+    }
+    *out = g;
+    return SG_OK;
+}
+
+int sg_graph_launch(sg_ctx *ctx, sg_graph *g) {
+    if (!ctx || !g || !g->exec) return SG_ERR_ARG;
+    if (ctx->capturing) return sg_fail(ctx, SG_ERR_ARG, "sg_graph_launch inside a capture");
+    SG_HIP(ctx, hipGraphLaunch(g->exec, ctx->stream));
+    return SG_OK;
+}
+
+int sg_graph_destroy(sg_ctx *ctx, sg_graph *g) {
+    if (!ctx) return SG_ERR_ARG;
+    if (!g) return SG_OK;
+    (void)hipStreamSynchronize(ctx->stream);  // a replay may still be running on the held workspaces
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    for (void *p : g->held) (void)sg_free(ctx, p);
+    delete g;
+    return SG_OK;
+}

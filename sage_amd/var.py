@@ -603,16 +603,52 @@ class Program:
     def __init__(self, ctx, targets):
         self.ctx = ctx
         self.calls = []
+        self.graph = None
         self._ev = _Evaluator(ctx, targets, record=self.calls)
         self.outputs = [self._ev.get(t) for t in targets]
 
-    def run(self):
+    def run_eager(self):
         h, check = self.ctx.handle, self.ctx.check
         for fn, args, _ in self.calls:
             rc = fn(h, *args)
             if rc:
                 check(rc)
         self.ctx.launches += len(self.calls)
+        return self.outputs
+
+    def capture(self):
+        """Record the launch sequence into a HIP graph (sg_graph_begin/end); `run()` then replays it with
+        one submission instead of one host call per operator.  The sequence has already run once in
+        the constructor, so every expression kernel is built and every buffer exists."""
+        if self.graph is not None:
+            return self
+        lib, h = self.ctx._lib, self.ctx.handle
+        self.ctx.check(lib.sg_graph_begin(h))
+        rc_call = 0
+        for fn, args, _ in self.calls:
+            rc_call = fn(h, *args)
+            if rc_call:
+                break
+        g = C.c_void_p()
+        rc_end = lib.sg_graph_end(h, C.byref(g))
+        if rc_call:
+            if not rc_end:
+                lib.sg_graph_destroy(h, g)
+            self.ctx.check(rc_call)
+        self.ctx.check(rc_end)
+        self.graph = g
+        return self
+
+    def release_graph(self):
+        if self.graph is not None and self.ctx.handle:
+            self.ctx._lib.sg_graph_destroy(self.ctx.handle, self.graph)
+        self.graph = None
+
+    def run(self):
+        if self.graph is None:
+            return self.run_eager()
+        self.ctx.check(self.ctx._lib.sg_graph_launch(self.ctx.handle, self.graph))
+        self.ctx.launches += 1
         return self.outputs
 
 

@@ -10,7 +10,7 @@ from sage_amd import var as V
 from sage_amd.bert import Bert, BertConfig, BertLayer
 from sage_amd.layers import load_params
 from sage_amd.resnet import ResNet, ResNetConfig
-from tests.util import REL_GEMM, close
+from tests.util import REL_GEMM, close, exact
 
 pytestmark = pytest.mark.gpu
 
@@ -187,3 +187,44 @@ def test_resnet18(ctx, fused):
     yo = O.resnet18_forward(ht(x), pod).numpy()
     assert y.shape == (3, 10)
     close(y, yo, REL_GEMM, "resnet vs oracle")
+
+
+@pytest.mark.parametrize("model", ["bert_layer", "resnet18"])
+def test_program_graph_replay(ctx, model):
+    """A compiled Program replayed as a HIP graph: several replays, with new input values, eager runs and
+    synchronisations between them, each compared with the eager result for the same input."""
+    say("graph replay", model)
+    rng = np.random.default_rng(11)
+    if model == "bert_layer":
+        n, l, e, heads, hdim = 2, 64, 128, 2, 256
+        p = bert_layer_params(rng, e, hdim, per_feature=True)
+        layer = BertLayer(BertConfig(e, 100, 512, hdim, 1, heads, 1e-12, 0.1, 2), reference_exact=False)
+        load_params(ctx, layer, layer_param_list(p))
+        xs = [rng.standard_normal((n, l, e)).astype(np.float32) for _ in range(3)]
+        xt = S.Tensor.from_numpy(ctx, xs[0])
+        out = layer.pass_(S.Var.new(xt), dev(ctx, np.ones((n, l), np.float32)))
+    else:
+        arrays, _ = resnet_arrays(rng, 1, 10)
+        net = ResNet(ResNetConfig.d18(1, 10))
+        load_params(ctx, net, arrays)
+        xs = [rng.uniform(0, 1, (16, 28, 28, 1)).astype(np.float32) for _ in range(3)]
+        xt = S.Tensor.from_numpy(ctx, xs[0])
+        out = net.pass_(S.Var.new(xt))
+    prog = S.Program(ctx, [out])
+    eager = []
+    for x in xs:
+        xt.copy_from_numpy(x)
+        eager.append(prog.run_eager()[0].numpy().copy())
+    assert not np.array_equal(eager[0], eager[1])
+    prog.capture()
+    try:
+        for rep in range(2):
+            for x, want in zip(xs, eager):
+                xt.copy_from_numpy(x)
+                got = prog.run()[0].numpy()
+                exact(got, want, f"graph replay {rep} vs eager")
+                ctx.sync()
+                xt.copy_from_numpy(xs[0])
+                exact(prog.run_eager()[0].numpy(), eager[0], "eager between replays")
+    finally:
+        prog.release_graph()

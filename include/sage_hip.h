@@ -239,6 +239,12 @@ int sg_gemm_kernel_name(sg_ctx *ctx, int64_t M, int64_t N, int64_t K, int64_t ba
 int sg_im2col(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, const int32_t ker[2],
               const int32_t stride[2], const int32_t pad[2], const int32_t dil[2]);
 
+/* Col2im::compute (conv.rs:405-500), the adjoint of sg_im2col used by Im2col::grad (conv.rs:275-287):
+ * x [N,OH,OW,KH,KW,C] dense -> out [N,H,W,C], each pixel the sum of the column entries taken from
+ * it (additions in the reference's order: column x outer, column y inner). */
+int sg_col2im(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, const int32_t ker[2],
+              const int32_t stride[2], const int32_t pad[2], const int32_t dil[2]);
+
 /* ---- fused row operators: compositions of ops/nn.rs ------------------------------------------ */
 
 /* softmax over the last axis (nn.rs:42-56) of (x + addend): one pass instead of reduce(max),

@@ -536,6 +536,18 @@ def im2col(x, ker, stride, pad, dil):  # conv.rs:188-226 ; pairs are [w, h]
     return y
 
 
+def col2im(x, img_size, ker, stride, pad, dil):  # conv.rs:229-264 ; img_size and pairs are [w, h]
+    ker, stride, pad, dil = _pair(ker), _pair(stride), _pair(pad), _pair(dil)
+    x = x.organize()
+    n, c = x.extents[0], x.extents[5]
+    y = HT.empty([n, img_size[1], img_size[0], c], x.dtype)
+    arr = lambda v: (C.c_int32 * 2)(*v)
+    xt, yt = x.ct(), y.ct()
+    if lib().or_col2im(C.byref(xt), C.byref(yt), arr(ker), arr(stride), arr(pad), arr(dil)):
+        raise RuntimeError("or_col2im failed")
+    return y
+
+
 def conv_2d(x, filt, stride, pad, dil):  # conv.rs:61-96
     kh, kw, cin, cout = filt.extents
     col = im2col(x, [kw, kh], stride, pad, dil)

@@ -648,6 +648,57 @@ int or_im2col(const sg_tensor *x, const sg_tensor *out, const int32_t ker[2], co
     return OR_OK;
 }
 
+/* ---------------------------------------------------------------------------------------------
+ * Col2im::compute (conv.rs:405-500).  Work-item = (img_y, img_x, c); the batch and the contributing
+ * columns are looped inside it, col_x outer and col_y inner (the order of the float additions).
+ * The reference tests ker_x against dilation_h and ker_y against dilation_w (conv.rs:463-465);
+ * kept as is, it only matters when the two dilations differ.  Pairs are {w, h}.
+ * ------------------------------------------------------------------------------------------- */
+int or_col2im(const sg_tensor *x, const sg_tensor *out, const int32_t ker[2], const int32_t stride[2],
+              const int32_t pad[2], const int32_t dil[2]) {
+    if (x->rank != 6 || out->rank != 4) return OR_ERR;
+    int batch = (int)x->extents[0], col_h = (int)x->extents[1], col_w = (int)x->extents[2], chan = (int)x->extents[5];
+    int img_h = (int)out->extents[1], img_w = (int)out->extents[2];
+    int ker_w = ker[0], ker_h = ker[1], stride_w = stride[0], stride_h = stride[1];
+    int padding_w = pad[0], padding_h = pad[1], dilation_w = dil[0], dilation_h = dil[1];
+    const float *col = (const float *)x->base;
+    float *img = (float *)out->base;
+    int col_offset = (int)x->offset, img_offset = (int)out->offset;
+    int gws = img_w * img_h * chan;
+#pragma omp parallel for schedule(static)
+    for (int gid = 0; gid < gws; ++gid) {
+        for (int n = 0; n < batch; ++n) {
+            int offset_img_batch = n * img_h * img_w * chan;
+            int offset_col_batch = n * col_h * col_w * ker_h * ker_w * chan;
+            int c = gid % chan;
+            int img_x = (gid / chan) % img_w;
+            int img_y = gid / (chan * img_w);
+            int img_x_pad = img_x + padding_w, img_y_pad = img_y + padding_h;
+            int ker_ew = (ker_w - 1) * dilation_w + 1, ker_eh = (ker_h - 1) * dilation_h + 1;
+            int col_x_start = (img_x_pad < ker_ew) ? 0 : (img_x_pad - ker_ew) / stride_w + 1;
+            int col_y_start = (img_y_pad < ker_eh) ? 0 : (img_y_pad - ker_eh) / stride_h + 1;
+            int col_x_end = img_x_pad / stride_w + 1 < col_w ? img_x_pad / stride_w + 1 : col_w;
+            int col_y_end = img_y_pad / stride_h + 1 < col_h ? img_y_pad / stride_h + 1 : col_h;
+            float val = 0.0f;
+            int offset_img = (img_y * img_w + img_x) * chan + img_offset;
+            for (int col_x = col_x_start; col_x < col_x_end; ++col_x) {
+                for (int col_y = col_y_start; col_y < col_y_end; ++col_y) {
+                    int ker_x = img_x_pad - col_x * stride_w;
+                    int ker_y = img_y_pad - col_y * stride_h;
+                    if (ker_x % dilation_h == 0 && ker_y % dilation_w == 0) {
+                        ker_x /= dilation_h;
+                        ker_y /= dilation_w;
+                        int offset_col = (((col_y * col_w + col_x) * ker_h + ker_y) * ker_w + ker_x) * chan + col_offset;
+                        val += col[offset_col_batch + offset_col + c];
+                    }
+                }
+            }
+            img[offset_img_batch + offset_img + c] = val;
+        }
+    }
+    return OR_OK;
+}
+
 int or_num_threads(void) {
 #ifdef _OPENMP
     extern int omp_get_max_threads(void);

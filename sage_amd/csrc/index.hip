@@ -114,6 +114,40 @@ __global__ void __launch_bounds__(256) im2col_kernel(const float *__restrict__ i
     }
 }
 
+// Col2im::compute (conv.rs:405-500): img[n,y,x,c] = sum of the column entries that im2col copied
+// from that pixel.  One thread per output element (the reference loops the batch inside a work-item);
+// the additions run col_x outer, col_y inner, as the reference's, so the sum is bit-identical to a
+// sequential restatement.  The reference tests ker_x against dilation_h and ker_y against dilation_w
+// (conv.rs:463-465); kept, it only matters when the two dilations differ.
+__global__ void __launch_bounds__(256) col2im_kernel(const float *__restrict__ col, float *__restrict__ img, uint32_t n_out, Im2colP p) {
+    const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
+    if (gid >= n_out) return;
+    const int c = gid % p.chan;
+    uint32_t t = gid / p.chan;
+    const int img_x = t % p.img_w;
+    t /= p.img_w;
+    const int img_y = t % p.img_h;
+    const int n = t / p.img_h;
+    const int img_x_pad = img_x + p.pad_w, img_y_pad = img_y + p.pad_h;
+    const int ker_ew = (p.ker_w - 1) * p.dil_w + 1, ker_eh = (p.ker_h - 1) * p.dil_h + 1;
+    const int col_x_start = img_x_pad < ker_ew ? 0 : (img_x_pad - ker_ew) / p.stride_w + 1;
+    const int col_y_start = img_y_pad < ker_eh ? 0 : (img_y_pad - ker_eh) / p.stride_h + 1;
+    const int col_x_end = min(img_x_pad / p.stride_w + 1, p.col_w);
+    const int col_y_end = min(img_y_pad / p.stride_h + 1, p.col_h);
+    const float *cb = col + (size_t)n * p.col_h * p.col_w * p.ker_h * p.ker_w * p.chan + c;
+    float val = 0.0f;
+    for (int col_x = col_x_start; col_x < col_x_end; ++col_x)
+        for (int col_y = col_y_start; col_y < col_y_end; ++col_y) {
+            int ker_x = img_x_pad - col_x * p.stride_w, ker_y = img_y_pad - col_y * p.stride_h;
+            if (ker_x % p.dil_h == 0 && ker_y % p.dil_w == 0) {
+                ker_x /= p.dil_h;
+                ker_y /= p.dil_w;
+                val += cb[(size_t)(((col_y * p.col_w + col_x) * p.ker_h + ker_y) * p.ker_w + ker_x) * p.chan];
+            }
+        }
+    img[gid] = val;
+}
+
 }  // namespace
 
 extern "C" int sg_fill_u32(sg_ctx *ctx, void *dst_dev, uint32_t pattern, uint64_t count) {
@@ -268,5 +302,32 @@ extern "C" int sg_im2col(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, 
         hipLaunchKernelGGL((im2col_kernel<1>), dim3((n + 255) / 256), dim3(256), 0, ctx->stream, img, col, n, p);
     }
     SG_CHECK_LAUNCH(ctx, "im2col");
+    return SG_OK;
+}
+
+extern "C" int sg_col2im(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, const int32_t ker[2], const int32_t stride[2],
+                         const int32_t pad[2], const int32_t dil[2]) {
+    if (!ctx || !ker || !stride || !pad || !dil) return SG_ERR_ARG;
+    int rc;
+    if ((rc = sg_validate_tensor(ctx, x, "sg_col2im x")) != SG_OK) return rc;
+    if ((rc = sg_validate_tensor(ctx, out, "sg_col2im out")) != SG_OK) return rc;
+    if (x->dtype != SG_FLOAT || out->dtype != SG_FLOAT) return sg_fail(ctx, SG_ERR_DTYPE, "sg_col2im: fp32 only");
+    if (x->rank != 6 || out->rank != 4) return sg_fail(ctx, SG_ERR_SHAPE, "sg_col2im: x must be [N,OH,OW,KH,KW,C], out [N,H,W,C] (conv.rs:243)");
+    if (!sg_is_dense(x) || !sg_is_dense(out)) return sg_fail(ctx, SG_ERR_SHAPE, "sg_col2im: x and out must be dense (conv.rs:244)");
+    for (int i = 0; i < 2; ++i)
+        if (ker[i] < 1 || stride[i] < 1 || pad[i] < 0 || dil[i] < 1) return sg_fail(ctx, SG_ERR_ARG, "sg_col2im: bad geometry");
+    Im2colP p;
+    p.batch = (int)out->extents[0]; p.img_h = (int)out->extents[1]; p.img_w = (int)out->extents[2]; p.chan = (int)out->extents[3];
+    p.ker_w = ker[0]; p.ker_h = ker[1]; p.stride_w = stride[0]; p.stride_h = stride[1];
+    p.pad_w = pad[0]; p.pad_h = pad[1]; p.dil_w = dil[0]; p.dil_h = dil[1];
+    p.col_h = (int)x->extents[1]; p.col_w = (int)x->extents[2];
+    if (x->extents[0] != p.batch || x->extents[3] != p.ker_h || x->extents[4] != p.ker_w || x->extents[5] != p.chan)
+        return sg_fail(ctx, SG_ERR_SHAPE, "sg_col2im: x is not [N,OH,OW,KH,KW,C] for this kernel size and output");
+    const int64_t total = sg_numel(out);
+    if (total >= (1ll << 32) || sg_numel(x) >= (1ll << 32)) return sg_fail(ctx, SG_ERR_SHAPE, "sg_col2im: more than 2^32 elements");
+    const float *col = (const float *)x->base + x->offset;
+    float *img = (float *)out->base + out->offset;
+    hipLaunchKernelGGL(col2im_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, col, img, (uint32_t)total, p);
+    SG_CHECK_LAUNCH(ctx, "col2im");
     return SG_OK;
 }

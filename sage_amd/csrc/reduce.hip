@@ -90,6 +90,31 @@ __global__ void __launch_bounds__(256) reduce_thread_kernel(const T *__restrict_
     y[gid] = acc;
 }
 
+// ---- column reduction: few contiguous outputs, a long strided reduced axis (bias gradients: the
+// sum over all rows of a [rows, C] matrix).  One thread per output would leave most of the chip idle
+// and read serially; here a workgroup takes 64 columns x a chunk of rows, its four wavefronts walk
+// alternate rows with coalesced 256-byte reads, and the per-chunk results are combined by a second,
+// small pass (in a fixed order: the result does not depend on scheduling).
+template <int OP, class T>
+__global__ void __launch_bounds__(256) reduce_cols_kernel(const T *__restrict__ x, T *__restrict__ part, uint32_t n_cols,
+                                                          uint32_t n_rows, uint32_t row_stride, uint32_t rows_per_chunk,
+                                                          uint32_t x_off) {
+    __shared__ T sh[4][64];
+    const uint32_t c = blockIdx.x * 64u + (threadIdx.x & 63u), ty = threadIdx.x >> 6;
+    const uint32_t r0 = blockIdx.y * rows_per_chunk, r1 = min(r0 + rows_per_chunk, n_rows);
+    T acc = identity<OP, T>();
+    if (c < n_cols) {
+        const T *p = x + x_off + c;
+        for (uint32_t r = r0 + ty; r < r1; r += 4) acc = combine<OP, T>(acc, p[(size_t)r * row_stride]);
+    }
+    sh[ty][threadIdx.x & 63u] = acc;
+    __syncthreads();
+    if (ty == 0 && c < n_cols) {
+        acc = combine<OP, T>(combine<OP, T>(sh[0][threadIdx.x], sh[1][threadIdx.x]), combine<OP, T>(sh[2][threadIdx.x], sh[3][threadIdx.x]));
+        part[(size_t)blockIdx.y * n_cols + c] = acc;
+    }
+}
+
 // ---- contiguous reduced span: ROWS_PER_BLOCK wavefronts, one row each, or one block per row ----
 template <int OP, class T, bool VEC4, bool BLOCK_PER_ROW>
 __global__ void __launch_bounds__(256) reduce_row_kernel(const T *__restrict__ x, T *__restrict__ y, uint32_t n_out,
@@ -492,6 +517,26 @@ int launch_reduce(sg_ctx *ctx, const sg_tensor *in, const sg_tensor *out, const 
             if (vec) hipLaunchKernelGGL((reduce_row_kernel<OP, T, true, false>), grid, dim3(256), 0, ctx->stream, x, y, (uint32_t)n_out, (uint32_t)in->offset, kept, len, ref_zero);
             else hipLaunchKernelGGL((reduce_row_kernel<OP, T, false, false>), grid, dim3(256), 0, ctx->stream, x, y, (uint32_t)n_out, (uint32_t)in->offset, kept, len, ref_zero);
         }
+    } else if (kept.n == 1 && kept.stride[0] == 1 && red.n == 1 && red_total >= 256 && n_out * 8 <= red_total * 64 && n_out <= 16384) {
+        // contiguous outputs, one long strided reduced axis: chunks of rows in parallel, then a combine pass
+        const uint32_t n_cols = (uint32_t)n_out, n_rows = (uint32_t)red_total;
+        const uint32_t col_tiles = (n_cols + 63) / 64;
+        uint32_t chunks = (4u * (uint32_t)(ctx->num_cus > 0 ? ctx->num_cus : 256) + col_tiles - 1) / col_tiles;
+        if (chunks > n_rows / 32) chunks = n_rows / 32;
+        if (chunks < 1) chunks = 1;
+        const uint32_t rows_per_chunk = (n_rows + chunks - 1) / chunks;
+        chunks = (n_rows + rows_per_chunk - 1) / rows_per_chunk;
+        void *ws = nullptr;
+        int rc = sg_alloc(ctx, (uint64_t)chunks * n_cols * sizeof(T), &ws);
+        if (rc != SG_OK) return rc;
+        hipLaunchKernelGGL((reduce_cols_kernel<OP, T>), dim3(col_tiles, chunks), dim3(256), 0, ctx->stream, x, (T *)ws, n_cols, n_rows,
+                           red.stride[0], rows_per_chunk, (uint32_t)in->offset);
+        Dims pk = kept, pr = red;
+        pr.ext[0] = chunks;
+        pr.stride[0] = n_cols;
+        hipLaunchKernelGGL((reduce_thread_kernel<OP, T>), dim3((n_cols + 255) / 256), dim3(256), 0, ctx->stream, (const T *)ws, y, n_cols, 0u, pk, pr, chunks, ref_zero);
+        SG_CHECK_LAUNCH(ctx, "reduce (columns)");
+        return sg_free(ctx, ws);  // later users of the block are ordered behind these kernels on the stream
     } else {
         dim3 grid((unsigned)((n_out + 255) / 256));
         hipLaunchKernelGGL((reduce_thread_kernel<OP, T>), grid, dim3(256), 0, ctx->stream, x, y, (uint32_t)n_out, (uint32_t)in->offset, kept, red, (uint32_t)red_total, ref_zero);

@@ -104,6 +104,11 @@ class Var:
             return self.value
         return evaluate(ctx, [self])[0]
 
+    def grad(self, y):
+        """Var::grad (var.rs:326-334): the gradient of `y` with respect to this variable."""
+        from .grad import grad
+        return grad(into_var(y), [self])[0]
+
     # ---- fluent API (var.rs:382-700)
     def copy(self): return unary_map(self, "copy")
     def abs(self): return unary_map(self, "abs")
@@ -508,6 +513,17 @@ def matmul_batched(x1, x2):
     return gemm_batched(a, b).view(ext)
 
 
+def matmul_batched_composed(x1, x2):
+    """matmul_batched exactly as the reference composes it (view -> gemm_batched -> view), whatever
+    the fusion setting; the gradient of the strided form is taken through this."""
+    on = _FUSION["on"]
+    _FUSION["on"] = False
+    try:
+        return matmul_batched(x1, x2)
+    finally:
+        _FUSION["on"] = on
+
+
 # ----------------------------------------------------------------------------- conv (ops/conv.rs)
 def _pair(v):
     return [int(v), int(v)] if isinstance(v, (int, np.integer)) else [int(v[0]), int(v[1])]
@@ -528,6 +544,16 @@ def im2col(x, ker_size, stride, padding, dilation):
     col = conv_size([w, h], ker, stride, pad, dil)
     return Var(Shape([n, col[1], col[0], ker[1], ker[0], c]), x.dtype, "im2col", [x],
                {"ker": ker, "stride": stride, "pad": pad, "dil": dil})
+
+
+def col2im(x, img_size, ker_size, stride, padding, dilation):
+    """conv.rs:229-264.  img_size and every pair are [w, h]; x is [N,OH,OW,KH,KW,C]."""
+    x = into_var(x).organize()
+    ker, stride, pad, dil = _pair(ker_size), _pair(stride), _pair(padding), _pair(dilation)
+    if x.rank != 6:
+        raise abi.ShapeError(abi.ERR_SHAPE, "col2im needs [N,OH,OW,KH,KW,C] (conv.rs:243)")
+    return Var(Shape([x.extents[0], img_size[1], img_size[0], x.extents[5]]), x.dtype, "col2im", [x],
+               {"img": list(img_size), "ker": ker, "stride": stride, "pad": pad, "dil": dil})
 
 
 def conv_2d(x, filt, stride, padding, dilation):
@@ -584,6 +610,13 @@ class _MapBuilder:
         self.prog.append((abi.EXPR_INPUT, self.keys[key], 0, 0))
 
 
+def evaluate_fresh(ctx, targets):
+    """Evaluate `targets` without keeping their tensors on the Vars (the reference clears ctx.data
+    between evaluations for the same effect, var.rs:121)."""
+    ev = _Evaluator(ctx, targets)
+    return [ev.get(t) for t in targets]
+
+
 def evaluate(ctx, targets):
     """Context::eval (context.rs:96-117): evaluate `targets`, keep their tensors on the Vars."""
     ev = _Evaluator(ctx, targets)
@@ -604,8 +637,17 @@ class Program:
         self.ctx = ctx
         self.calls = []
         self.graph = None
+        self.targets = list(targets)
         self._ev = _Evaluator(ctx, targets, record=self.calls)
         self.outputs = [self._ev.get(t) for t in targets]
+
+    def bind(self):
+        """Keep each target's output tensor on its Var (the role of ctx.data after Program::exec,
+        session.rs:657-664): later expressions, e.g. an optimizer's, can then use the targets as data.
+        The tensors are rewritten in place by every run."""
+        for t, o in zip(self.targets, self.outputs):
+            t.value = o
+        return self
 
     def run_eager(self):
         h, check = self.ctx.handle, self.ctx.check
@@ -904,6 +946,17 @@ class _Evaluator:
         arr = lambda p: (C.c_int32 * 2)(*p)
         xc, yc = x.c(), y.c()
         self.call(self.lib.sg_im2col, C.byref(xc), C.byref(yc), arr(a["ker"]), arr(a["stride"]), arr(a["pad"]), arr(a["dil"]))
+        return y
+
+    def _ev_col2im(self, v):
+        x = self.get(v.inputs[0])
+        if not x.is_dense():
+            x = self.run_copy(x)
+        y = self.out(v.extents, v.dtype)
+        a = v.attrs
+        arr = lambda p: (C.c_int32 * 2)(*p)
+        xc, yc = x.c(), y.c()
+        self.call(self.lib.sg_col2im, C.byref(xc), C.byref(yc), arr(a["ker"]), arr(a["stride"]), arr(a["pad"]), arr(a["dil"]))
         return y
 
     # ---- GEMM family, with optional epilogue and destination layout

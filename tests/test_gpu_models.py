@@ -61,7 +61,8 @@ def layer_param_list(p):
 
 def torch_bert_layer(x, mask, p, heads, act, eps):
     import torch
-    t = lambda a: torch.from_numpy(np.asarray(a)).double()
+    as_tensor = torch.is_tensor(x)  # tensors pass through (autograd use); arrays are converted
+    t = lambda a: a if torch.is_tensor(a) else torch.from_numpy(np.asarray(a)).double()
     x = t(x)
     n, l, e = x.shape
     d = e // heads
@@ -80,7 +81,8 @@ def torch_bert_layer(x, mask, p, heads, act, eps):
     h1 = lnorm(lin(a, p["wo"], p["bo"]) + x, p["ln1_g"], p["ln1_b"])
     u = lin(h1, p["w1"], p["b1"])
     u = torch.relu(u) if act == "relu" else 0.5 * u * (1 + torch.erf(u / np.sqrt(2.0)))
-    return lnorm(lin(u, p["w2"], p["b2"]) + h1, p["ln2_g"], p["ln2_b"]).numpy()
+    out = lnorm(lin(u, p["w2"], p["b2"]) + h1, p["ln2_g"], p["ln2_b"])
+    return out if as_tensor else out.numpy()
 
 
 @pytest.mark.parametrize("reference_exact", [True, False], ids=["reference_exact", "gelu_config"])

@@ -199,6 +199,8 @@ def test_fused_map_equals_unfused(ctx):
 RED_CASES = [
     ((8, 1024), [1]), ((8, 1024), [0]), ((5, 37), [1]), ((3, 5000), [1]), ((64, 9, 32), [1]),
     ((2, 3, 2, 3, 2), [0, 2, 3]), ((6, 7, 8), [0, 1, 2]), ((4, 6, 10), [2, 0]), ((128, 128), [1]), ((1, 7), [0]),
+    # few contiguous outputs, long strided reduced axis (bias gradients): chunked column path
+    ((5000, 70), [0]), ((6272, 64), [0]), ((3, 400, 513), [0, 1]), ((300, 16), [0]),
 ]
 
 
@@ -243,6 +245,9 @@ def test_reduce_strided_and_int(ctx):
     i = rng.integers(-20, 20, (9, 33)).astype(np.int32)
     exact(dev(ctx, i).sum(1).eval(ctx).numpy(), O.rsum(ht(i), 1).numpy(), "int sum")
     exact(dev(ctx, i).max(0).eval(ctx).numpy(), O.rmax(ht(i), 0).numpy(), "int max")
+    j = rng.integers(-20, 20, (4000, 40)).astype(np.int32)
+    exact(dev(ctx, j).sum(0).eval(ctx).numpy(), O.rsum(ht(j), 0).numpy(), "int column sum")
+    exact(dev(ctx, j).min(0).eval(ctx).numpy(), O.rmin(ht(j), 0).numpy(), "int column min")
 
 
 @pytest.mark.parametrize("shape,axis", [((2, 3, 4), 1), ((64, 1000), 1), ((64, 1000), 0), ((5, 7, 300), 2), ((9, 64), 1), ((3, 1), 1)])

@@ -223,3 +223,34 @@ def test_map_dtype_rules_and_errors():
     assert source([UN("exp"), INP(0)], [desc([4, 5])], f)[0] == abi.ERR_SHAPE    # ops.rs:174
     assert source([UN("exp"), INP(0)], [f], desc([4, 4], [1, 4]))[0] == abi.ERR_SHAPE  # output not dense
     assert source([UN("exp"), INP(0)], [desc([4, 4], dtype=abi.LONG)], f)[0] == abi.ERR_DTYPE
+
+
+def test_gradient_graph_construction():
+    """grad (var.rs:56-103) only builds graphs: no device is needed to check its structure."""
+    from sage_amd import nn
+    from sage_amd.grad import grad, grad_param, t_order
+    from sage_amd.resnet import ResNet, ResNetConfig
+    from sage_amd.tensor import UINT
+    from sage_amd.var import Var
+    x = Var.empty([3, 4])
+    y = (x.exp() * x).sum([1], False)
+    assert t_order(x) == 0 and t_order(y) == 3  # exp -> mul -> reduce (ops.rs:262-310)
+    (gx,) = grad(y, [x])
+    assert gx.extents == [3, 4] and gx.op == "binary" and gx.attrs["name"] == "add"  # two consumers of x: summed
+    with pytest.raises(KeyError):
+        grad(y, [Var.empty([2])])
+    model = ResNet(ResNetConfig.d18(1, 10))
+    img, lab = Var.empty([4, 28, 28, 1]), Var.empty([4, 1], UINT)
+    loss = nn.softmax_cross_entropy(model.pass_(img), lab).mean(0, False)
+    g = grad_param(loss, model)
+    assert len(g) == 42 and all(gv.extents == p.extents for p, gv in g.items())
+    ops = set()
+    stack, seen = list(g.values()), set()
+    while stack:
+        v = stack.pop()
+        if id(v) in seen:
+            continue
+        seen.add(id(v))
+        ops.add(v.op)
+        stack.extend(v.inputs)
+    assert "col2im" in ops and "gemm" in ops and "cond" in ops  # conv backward, dense backward, max-pool backward

@@ -145,6 +145,21 @@ def test_im2col(golden):
     close(O.im2col(T(g("x")), [3, 2], [1, 1], [0, 0], [1, 1]).numpy(), g("y_gt"), 1e-3)
 
 
+def test_col2im(golden):
+    """conv.rs:699-990: [2,4,2,2,3,3] -> [2,5,4,3], img (w,h) = [4,5], ker (w,h) = [3,2]; plus the adjoint
+    identity <im2col(x), c> = <x, col2im(c)> that any col2im must satisfy, with stride, padding and dilation."""
+    g = lambda n: golden("src/ops/conv.rs", "test_col2im", n)
+    close(O.col2im(T(g("x")), [4, 5], [3, 2], [1, 1], [0, 0], [1, 1]).numpy(), g("y_gt"), 1e-3)
+    rng = np.random.default_rng(0)
+    for (h, w, c, ker, stride, pad, dil) in [(9, 7, 3, [3, 3], [2, 2], [1, 1], [1, 1]), (11, 10, 2, [3, 2], [2, 1], [0, 1], [2, 2])]:
+        x = rng.standard_normal((2, h, w, c)).astype(np.float32)
+        xc = O.im2col(T(x), ker, stride, pad, dil).numpy()
+        col = rng.standard_normal(xc.shape).astype(np.float32)
+        back = O.col2im(T(col), [w, h], ker, stride, pad, dil).numpy()
+        lhs, rhs = float((xc.astype(np.float64) * col).sum()), float((x.astype(np.float64) * back).sum())
+        assert abs(lhs - rhs) < 1e-3 * max(1.0, abs(lhs))
+
+
 def test_conv2d(golden):
     """conv.rs:1014-1534: [1,5,5,4] * [3,3,4,8], pad 1"""
     g = lambda n: golden("src/ops/conv.rs", "test_conv2d", n)

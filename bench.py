@@ -322,9 +322,59 @@ def run_kernel_workload(a):
     print(json.dumps(res))
 
 
+def run_train_workload(a):
+    """One training step of examples/train.rs: ResNet-18 on [B,28,28,1] -> mean softmax-CE -> grad_param -> Adam,
+    as two replayed programs (forward+backward, optimizer update)."""
+    import sage_amd as S
+    from sage_amd import nn, optim
+    from sage_amd.grad import grad_param
+    ctx = S.Context(0)
+    rng = np.random.default_rng(4)
+    batch = a.batch if a.batch != 32 else 128
+    model, arrays, x_host, logits = build_resnet18(ctx, batch, rng)
+    labels = rng.integers(0, 10, (batch, 1)).astype(np.int32)
+    loss = nn.softmax_cross_entropy(logits, S.Var.new(S.Tensor.from_numpy(ctx, labels))).mean(0, False)
+    grads = grad_param(loss, model)
+    prog = S.Program(ctx, list(grads.values()) + [loss]).bind()
+    opt = optim.Adam(1e-4)
+    opt.init(ctx)
+    opt.update(grads, ctx)           # the reference's first update only creates the (zero) moments
+    upd = opt.compile(grads, ctx)
+    use_graph = a.graph != "off"
+    if use_graph:
+        prog.capture()
+        upd.capture()
+    gflops = sum(f for _, _, f, _ in gemm_calls(ctx, prog))
+    for _ in range(a.warmup):
+        prog.run()
+        upd.run()
+    ctx.sync()
+    loss0 = float(prog.outputs[-1].numpy()[0])
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        prog.run()
+        upd.run()
+    ctx.sync()
+    dt = time.perf_counter() - t0
+    loss1 = float(prog.outputs[-1].numpy()[0])
+    if not (np.isfinite(loss1) and loss1 < loss0):
+        raise SystemExit(f"training on a fixed batch did not reduce the loss ({loss0} -> {loss1})")
+    ms = dt / a.steps * 1e3
+    achieved = gflops / (ms * 1e-3) / 1e12
+    res = {"metric": f"ResNet-18 train step images/sec (b{batch},28x28x1,fp32,Adam)", "value": batch / (ms * 1e-3), "unit": "images/s",
+           "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": f"resnet18_train_b{batch}_28x28x1_fp32_adam", "replay": "hip_graph" if use_graph else "eager",
+                      "launches_per_step": len(prog.calls) + len(upd.calls), "loss_first": loss0, "loss_last": loss1},
+           "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                        "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+                        "kernel": "all GEMM launches of the step over the whole step time (the step is launch- and HBM-bound, no single dominant kernel)"}}
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="bert", help="bert (default, the headline metric) | resnet18 | softmax_ce | map_exp_sub | "
+    ap.add_argument("--workload", default="bert", help="bert (default, the headline metric) | resnet18 | resnet18_train | softmax_ce | map_exp_sub | "
                     "bias_residual | layer_norm | softmax | reduce_sum | gemm_bias")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
@@ -341,6 +391,8 @@ def main():
         print("bench.py measures one GPU: every box in this run has one MI355X and the hot path uses no "
               "collectives; run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if a.workload == "resnet18_train":
+        return run_train_workload(a)
     if a.workload not in ("bert", "resnet18"):
         return run_kernel_workload(a)
 

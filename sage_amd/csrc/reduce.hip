@@ -521,7 +521,8 @@ int launch_reduce(sg_ctx *ctx, const sg_tensor *in, const sg_tensor *out, const 
         // contiguous outputs, one long strided reduced axis: chunks of rows in parallel, then a combine pass
         const uint32_t n_cols = (uint32_t)n_out, n_rows = (uint32_t)red_total;
         const uint32_t col_tiles = (n_cols + 63) / 64;
-        uint32_t chunks = (4u * (uint32_t)(ctx->num_cus > 0 ? ctx->num_cus : 256) + col_tiles - 1) / col_tiles;
+        uint32_t chunks = (2u * (uint32_t)(ctx->num_cus > 0 ? ctx->num_cus : 256) + col_tiles - 1) / col_tiles;
+        if (chunks > 128) chunks = 128;  // the combine pass walks the chunks serially per output
         if (chunks > n_rows / 32) chunks = n_rows / 32;
         if (chunks < 1) chunks = 1;
         const uint32_t rows_per_chunk = (n_rows + chunks - 1) / chunks;

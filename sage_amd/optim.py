@@ -40,11 +40,31 @@ def _assign(param, new_tensor, ctx):
                                 C.c_void_p(new_tensor.buf.ptr + new_tensor.shape.offset * 4), old.size() * 4))
 
 
+def _compile(ctx, pairs):
+    """pairs: [(expression Var, destination Tensor)].  One Program that evaluates every expression and then
+    copies each result into its destination; building it performs the step once."""
+    from .var import Program
+    prog = Program(ctx, [e for e, _ in pairs])
+    lib = ctx._lib
+    for out, (_, dest) in zip(prog.outputs, pairs):
+        args = (C.c_void_p(dest.buf.ptr + dest.shape.offset * 4), C.c_void_p(out.buf.ptr + out.shape.offset * 4), C.c_uint64(dest.size() * 4))
+        ctx.check(lib.sg_memcpy_d2d(ctx.handle, *args))
+        prog.calls.append((lib.sg_memcpy_d2d, args, [out, dest]))
+    return prog
+
+
 class Optimizer:
     def init(self, ctx):
         raise NotImplementedError
 
     def update(self, grads, ctx):
+        raise NotImplementedError
+
+    def compile(self, grads, ctx):
+        """The update of `update(grads, ctx)` as a replayable `Program` (which can also be captured into a
+        HIP graph): same expressions, evaluated once per `run()` on fixed buffers, with the state and the
+        parameters rewritten in place.  Building it performs one update.  The reference has no
+        counterpart: its optimizers rebuild and evaluate their expressions on every step."""
         raise NotImplementedError
 
 
@@ -77,6 +97,16 @@ class Sgd(Optimizer):
                 self.g[id(grad)] = g.eval(ctx)
                 g = Var.new(self.g[id(grad)])
             _assign(param, (param - g * self.lr).eval(ctx), ctx)
+
+    def compile(self, grads, ctx):
+        if self.momentum != 0.0:
+            raise KeyError("Sgd with momentum fails in the reference (optim.rs:67-69)")
+        pairs = []
+        for param, grad in grads.items():
+            gv = Var.new(_value(grad, ctx))
+            g = gv + param * self.weight_decay if self.weight_decay != 0.0 else gv
+            pairs.append((param - g * self.lr, param.value))
+        return _compile(ctx, pairs)
 
 
 class Adam(Optimizer):
@@ -120,3 +150,22 @@ class Adam(Optimizer):
             v_hat = v_t / (-scalar(self.beta2, [1]).pow(t) + 1.0)
             _assign(param, (param - m_hat * self.lr / (v_hat.sqrt() + self.eps)).eval(ctx), ctx)
         self.t = (t + 1.0).eval(ctx)
+
+    def compile(self, grads, ctx):
+        if self.t is None or any(id(g) not in self.m_t for g in grads.values()):
+            raise RuntimeError("Adam.compile needs the state of every gradient: call update() once first "
+                               "(the first update creates all-zero moments, optim.rs:149-163)")
+        t = Var.new(self.t)
+        pairs = []
+        for param, grad in grads.items():
+            gv = Var.new(_value(grad, ctx))
+            g = gv + param * self.weight_decay if self.weight_decay != 0.0 else gv
+            key = id(grad)
+            m_t = Var.new(self.m_t[key]) * self.beta1 + g * (1.0 - self.beta1)
+            v_t = Var.new(self.v_t[key]) * self.beta2 + g.pow(2.0) * (1.0 - self.beta2)
+            m_hat = m_t / (-scalar(self.beta1, [1]).pow(t) + 1.0)
+            v_hat = v_t / (-scalar(self.beta2, [1]).pow(t) + 1.0)
+            pairs += [(m_t, self.m_t[key]), (v_t, self.v_t[key]),
+                      (param - m_hat * self.lr / (v_hat.sqrt() + self.eps), param.value)]
+        pairs.append((t + 1.0, self.t))
+        return _compile(ctx, pairs)

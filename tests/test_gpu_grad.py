@@ -340,6 +340,30 @@ def test_resnet18_training_step_vs_torch_and_adam(ctx):
             exact(params[0].value.numpy(), arrays[0], "the first Adam update leaves the weights as they were")
     assert not np.array_equal(params[0].value.numpy(), arrays[0])
 
+    # the same update as a replayable Program: building it is update 4, every run() one more; also as a HIP graph
+    def numpy_step(gs):
+        nonlocal t
+        for i, g in enumerate(gs):
+            m[i] = m[i] * 0.9 + g * (1.0 - 0.9)
+            v[i] = v[i] * 0.999 + g ** 2 * (1.0 - 0.999)
+            w[i] = w[i] - (m[i] / (1.0 - 0.9 ** t)) * 1e-3 / (np.sqrt(v[i] / (1.0 - 0.999 ** t)) + 1e-8)
+        t += 1.0
+
+    prog.run()
+    numpy_step([o.numpy().astype(np.float64) for o in prog.outputs[:-1]])
+    upd = opt.compile(grads, ctx)
+    for use_graph in (False, True):
+        if use_graph:
+            upd.capture()
+        for _ in range(2):
+            prog.run()
+            numpy_step([o.numpy().astype(np.float64) for o in prog.outputs[:-1]])
+            upd.run()
+    upd.release_graph()
+    for i, p in enumerate(params):
+        close(p.value.numpy(), w[i], 3e-3, f"compiled updates, parameter {i}")
+    close(opt.t.numpy(), np.array([t]), 1e-6, "step counter")
+
 
 def test_bert_layer_gradients_vs_torch(ctx):
     say("bert layer grads")

@@ -211,7 +211,8 @@ typedef struct sg_gemm_epilogue {
     const sg_tensor *residual; /* same extents as C, last stride 1, or NULL */
 } sg_gemm_epilogue;
 
-/* Gemm::compute_direct (gemm.rs:176-250): a, b, c are rank 2; (m,k,n) are taken from the extents
+/* (A long-K product with few output tiles uses a workspace from the context allocator: SG_ERR_OOM when it does not fit.)
+ * Gemm::compute_direct (gemm.rs:176-250): a, b, c are rank 2; (m,k,n) are taken from the extents
  * as gemm.rs:190-217 does for the four transpose modes; ld = strides[0] and the inner stride must
  * be 1 (the reference organizes its inputs first, gemm.rs:111-112).  fp32 only. */
 int sg_gemm(sg_ctx *ctx, int transpose_a, int transpose_b, const sg_tensor *a, const sg_tensor *b,

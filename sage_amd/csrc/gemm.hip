@@ -516,8 +516,14 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
     const int nsplit = choose_split(ctx->num_cus, (int64_t)p.tiles_m * p.tiles_n * batch, p.K, &k_chunk);
     if (nsplit > 1) {
         const int64_t slice = (int64_t)batch * p.M * p.N;
+        // The workspace comes from the context's allocator and counts against its capacity.  When it
+        // does not fit the call fails with SG_ERR_OOM like any other allocation (the caller's
+        // eviction loop, session.rs:259-325, frees memory and calls again) instead of silently taking
+        // the single-pass kernel, whose rounding differs: the same call always gives the same bits.
         void *ws = nullptr;
-        if (sg_alloc(ctx, (uint64_t)nsplit * slice * sizeof(float), &ws) == SG_OK) {
+        const int rc_ws = sg_alloc(ctx, (uint64_t)nsplit * slice * sizeof(float), &ws);
+        if (rc_ws != SG_OK) return rc_ws;
+        {
             GemmP q = p;  // first pass: raw partial products into the workspace
             q.C = (float *)ws;
             q.c_sm = p.N; q.c_sb1 = (int64_t)p.M * p.N; q.c_sb0 = q.c_sb1 * p.nb1; q.c_sz = slice;
@@ -537,7 +543,6 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
             // the block returns to the context's cache; later users are ordered behind these kernels on the stream
             return sg_free(ctx, ws);
         }
-        // no room for the workspace: fall through to the single-pass kernel
     }
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
     if (needs_guard(p, BM, BN)) launch_layouts<BM, BN, WAVES_M, true>(ctx, p, grid, a_kc, b_nc);

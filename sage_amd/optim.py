@@ -20,7 +20,7 @@ Reference behaviour that is kept because results would differ otherwise:
 import ctypes as C
 
 from .tensor import Tensor
-from .var import Var, evaluate, scalar
+from .var import Var, evaluate, params_changed, scalar
 
 
 def _value(grad, ctx):
@@ -35,6 +35,7 @@ def _assign(param, new_tensor, ctx):
     if old is None or not old.is_dense() or old.extents != new_tensor.extents or not new_tensor.is_dense():
         param.set(new_tensor)
         return
+    params_changed()
     lib = ctx._lib
     ctx.check(lib.sg_memcpy_d2d(ctx.handle, C.c_void_p(old.buf.ptr + old.shape.offset * 4),
                                 C.c_void_p(new_tensor.buf.ptr + new_tensor.shape.offset * 4), old.size() * 4))
@@ -50,6 +51,8 @@ def _compile(ctx, pairs):
         args = (C.c_void_p(dest.buf.ptr + dest.shape.offset * 4), C.c_void_p(out.buf.ptr + out.shape.offset * 4), C.c_uint64(dest.size() * 4))
         ctx.check(lib.sg_memcpy_d2d(ctx.handle, *args))
         prog.calls.append((lib.sg_memcpy_d2d, args, [out, dest]))
+    prog.changes_params = True
+    params_changed()
     return prog
 
 

@@ -16,6 +16,11 @@ _NP_OF = {FLOAT: np.float32, INT: np.int32, UINT: np.uint32}
 _DT_OF = {np.dtype(np.float32): FLOAT, np.dtype(np.int32): INT, np.dtype(np.uint32): UINT}
 
 
+# Bumped whenever existing device data may have been rewritten in place from the host side or by an
+# optimizer; caches of data derived from parameters (var.py) compare against it.
+_PARAM_EPOCH = [0]
+
+
 class Context:
     """Context::with_device (context.rs:43-52).  capacity=None: bounded by the device only;
     capacity=abi.REFERENCE_CAPACITY_BYTES reproduces the reference's 1000 MiB allocator cap."""
@@ -116,6 +121,7 @@ class Tensor:
             raise abi.ShapeError(abi.ERR_SHAPE, "copy_from_numpy needs a dense tensor of the same extents")
         dst = C.c_void_p(self.buf.ptr + self.shape.offset * 4)
         ctx.check(ctx._lib.sg_memcpy_h2d(ctx.handle, dst, a.ctypes.data_as(C.c_void_p), a.nbytes))
+        _PARAM_EPOCH[0] += 1
 
     def numpy(self):
         """Blocking read of the whole buffer, then the strided view is taken on the host."""

@@ -31,6 +31,16 @@ _FUSION = {"on": True}
 THRES = 5  # session.rs:75
 
 
+# Parameters may be rewritten in place (optimizers do); derived data that the evaluator caches, the
+# concatenated weights of sibling Dense layers, is rebuilt when this counter has moved since it was made.
+from .tensor import _PARAM_EPOCH  # noqa: E402  (shared counter, also bumped by Tensor.copy_from_numpy)
+
+
+def params_changed():
+    """Tell cached derived data that parameter values may have changed."""
+    _PARAM_EPOCH[0] += 1
+
+
 def set_fusion(on):
     _FUSION["on"] = bool(on)
 
@@ -73,6 +83,7 @@ class Var:
         self.value = tensor
         self.shape = tensor.shape.copy()
         self.dtype = tensor.dtype
+        params_changed()
 
     def name(self, label):
         self.label = label
@@ -610,6 +621,15 @@ class _MapBuilder:
         self.prog.append((abi.EXPR_INPUT, self.keys[key], 0, 0))
 
 
+def refresh_derived(ctx, entries):
+    """Re-run the calls that build cached derived data when parameters changed since they last ran."""
+    for e in entries:
+        if e["epoch"] != _PARAM_EPOCH[0]:
+            for fn, args, _ in e["calls"]:
+                ctx.check(fn(ctx.handle, *args))
+            e["epoch"] = _PARAM_EPOCH[0]
+
+
 def evaluate_fresh(ctx, targets):
     """Evaluate `targets` without keeping their tensors on the Vars (the reference clears ctx.data
     between evaluations for the same effect, var.rs:121)."""
@@ -640,6 +660,8 @@ class Program:
         self.targets = list(targets)
         self._ev = _Evaluator(ctx, targets, record=self.calls)
         self.outputs = [self._ev.get(t) for t in targets]
+        self.derived = self._ev.derived
+        self.changes_params = False  # set by optimizers: every run rewrites parameter values
 
     def bind(self):
         """Keep each target's output tensor on its Var (the role of ctx.data after Program::exec,
@@ -651,6 +673,9 @@ class Program:
 
     def run_eager(self):
         h, check = self.ctx.handle, self.ctx.check
+        refresh_derived(self.ctx, self.derived)
+        if self.changes_params:
+            params_changed()
         for fn, args, _ in self.calls:
             rc = fn(h, *args)
             if rc:
@@ -689,6 +714,9 @@ class Program:
     def run(self):
         if self.graph is None:
             return self.run_eager()
+        refresh_derived(self.ctx, self.derived)
+        if self.changes_params:
+            params_changed()
         self.ctx.check(self.ctx._lib.sg_graph_launch(self.ctx.handle, self.graph))
         self.ctx.launches += 1
         return self.outputs
@@ -746,6 +774,14 @@ class _Evaluator:
         self.keep = {}  # id -> Var, keeps nodes alive while ids are used as keys
         self.record = record
         self.keepalive = []
+        # Memory behaviour of Program::exec (session.rs:208-330) for a one-off evaluation: intermediates
+        # are dropped once every consumer has run, and when an allocation runs out of memory the cheapest
+        # retained intermediate (recompute time per byte) is dropped and recomputed on demand later.  A
+        # recorded Program keeps every buffer instead: its launches are replayed on them.
+        self.derived = []  # cached derived-data entries this evaluation relies on (see refresh_derived)
+        self.release = record is None
+        self.computed = set()
+        self.evictions = 0
 
     # ---- helpers
     def n_users(self, v):
@@ -764,19 +800,91 @@ class _Evaluator:
             t = getattr(self, "_ev_" + v.op)(v)
             self.memo[id(v)] = t
             self.keep[id(v)] = v
+            self.computed.add(id(v))
+            if self.release:
+                self._release_consumed(v)
         return t
+
+    def _finished(self, u, cache):
+        """Every path from u to a target passes through a node that has been computed."""
+        k = id(u)
+        if k in self.computed or k in self.memo or u.value is not None:
+            return True
+        if k in self.targets:
+            return False
+        if k not in cache:
+            cache[k] = False
+            us = self.users.get(k, ())
+            cache[k] = bool(us) and all(self._finished(w, cache) for w in us)
+        return cache[k]
+
+    def _release_consumed(self, v):
+        """Drop the tensors that the evaluation of v consumed and nobody else still needs: the retained
+        nodes reachable from v through nodes that were fused away rather than materialised."""
+        cache, seen, stack = {}, set(), list(v.inputs)
+        while stack:
+            n = stack.pop()
+            if id(n) in seen or n.value is not None:
+                continue
+            seen.add(id(n))
+            if id(n) in self.memo:
+                if id(n) not in self.targets and all(self._finished(u, cache) for u in self.users.get(id(n), ())):
+                    del self.memo[id(n)]
+            else:
+                stack.extend(n.inputs)
+
+    @staticmethod
+    def _recompute_cost(v):
+        """Rough time to recompute one node from its inputs (the reference measures Routine::exec_time)."""
+        n = float(v.size())
+        if v.op in GEMM_OPS:
+            a = v.inputs[0]
+            return 2.0 * n * a.extents[-1] / 1e5 + 10.0
+        if v.op in ("reduce", "reduce_arg", "softmax", "softmax_ce", "layer_norm"):
+            return float(v.inputs[0].size()) / 2e3 + 5.0
+        return n / 2e3 + 3.0
+
+    def _evict(self, needed):
+        """session.rs:259-325: free at least `needed` bytes by dropping retained intermediates, cheapest
+        recompute time per byte first.  Tensors still referenced by the operator being evaluated stay
+        alive whatever is dropped here (the reference's `lock` set plays that role)."""
+        start = self.ctx.mem_stats()["used"]
+        cands = [self.keep[k] for k in self.memo if k not in self.targets and k in self.keep and self.keep[k].value is None
+                 and self.keep[k].op != "data"]
+        cands.sort(key=lambda n: (self._recompute_cost(n) + 1.0) / (n.size() + 1.0))
+        for n in cands:
+            del self.memo[id(n)]
+            self.computed.discard(id(n))
+            self.evictions += 1
+            if start - self.ctx.mem_stats()["used"] >= needed:
+                return True
+        if start - self.ctx.mem_stats()["used"] >= needed:
+            return True
+        self.ctx.__dict__.get("_wide_weights", {}).clear()  # rebuilt on demand; recorded Programs keep their own
+        return start - self.ctx.mem_stats()["used"] >= needed
 
     def call(self, fn, *args):
         """Issue one operator launch through the C ABI; remember it when a Program is being compiled.
         The epilogue struct keeps pointers into `keepalive` objects, so those are stored too."""
         self.ctx.launches += 1
-        self.ctx.check(fn(self.ctx.handle, *args))
+        while True:
+            try:
+                self.ctx.check(fn(self.ctx.handle, *args))
+                break
+            except abi.OutOfMemory as e:  # a workspace inside the library did not fit
+                if not self.release or not self._evict(e.needed or 1):
+                    raise
         if self.record is not None:
             self.record.append((fn, args, list(self.keepalive)))
         self.keepalive = []
 
     def out(self, extents, dtype):
-        return Tensor.uninit(self.ctx, extents, dtype)
+        while True:
+            try:
+                return Tensor.uninit(self.ctx, extents, dtype)
+            except abi.OutOfMemory as e:
+                if not self.release or not self._evict(e.needed or 1):
+                    raise
 
     # ---- layout operators: descriptor rewrites on the evaluated tensor
     def _ev_reshape(self, v):
@@ -1288,12 +1396,17 @@ class _Evaluator:
             wcat, bcat = self.out([K, ntot], FLOAT), self.out([ntot], FLOAT)
             wi = (abi.sg_tensor * len(ws))(*[w.c() for w in ws])
             wc = wcat.c()
-            self.ctx.check(self.lib.sg_concat(self.ctx.handle, 1, wi, len(ws), C.byref(wc)))
             bi = (abi.sg_tensor * len(bs))(*[b.with_shape(Shape([b.size()], [1], b.shape.offset)).c() for b in bs])
             bc = bcat.c()
-            self.ctx.check(self.lib.sg_concat(self.ctx.handle, 0, bi, len(bs), C.byref(bc)))
-            cache[key] = (wcat, bcat, ws, bs)  # the sources are kept so their pointers stay unique
-        wcat, bcat = cache[key][0], cache[key][1]
+            # the two concatenations, kept as replayable calls: they run again whenever parameters have
+            # been rewritten since (an optimizer step), for this evaluation and for any recorded Program
+            calls = [(self.lib.sg_concat, (1, wi, len(ws), C.byref(wc)), [wi, wc]), (self.lib.sg_concat, (0, bi, len(bs), C.byref(bc)), [bi, bc])]
+            cache[key] = {"w": wcat, "b": bcat, "src": (ws, bs), "calls": calls, "epoch": None}  # sources kept: pointers stay unique
+        entry = cache[key]
+        refresh_derived(self.ctx, [entry])
+        if self.record is not None and entry not in self.derived:
+            self.derived.append(entry)
+        wcat, bcat = entry["w"], entry["b"]
         a = self.get(a_node)
         if not a.is_dense():
             a = self.run_copy(a)

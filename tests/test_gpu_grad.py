@@ -405,3 +405,35 @@ def test_sgd_plain_and_reference_momentum_bug(ctx):
     close(p.value.numpy(), w0 - 0.1 * w0, 1e-6, "w - lr * w")
     with pytest.raises(KeyError):  # optim.rs:67-69: the reference indexes a missing momentum entry
         optim.Sgd(0.1, momentum=0.9).update({p: grad(loss, [p])[0]}, ctx)
+
+
+def test_fused_sibling_dense_follows_parameter_updates(ctx):
+    """q/k/v projections sharing an input run as one GEMM on concatenated weights.  The concatenation is derived
+    data: after the parameters are rewritten in place (an optimizer step, a host write) a replayed Program and
+    a fresh evaluation must both see the new weights."""
+    say("wide weights after updates")
+    rng = np.random.default_rng(43)
+    n, l, e, heads, hdim = 2, 16, 64, 2, 128
+    p = bert_layer_params(rng, e, hdim, per_feature=True)
+    layer = BertLayer(BertConfig(e, 100, 512, hdim, 1, heads, 1e-12, 0.1, 2), reference_exact=False)
+    load_params(ctx, layer, layer_param_list(p))
+    x = rng.standard_normal((n, l, e)).astype(np.float32)
+    mask = np.ones((n, l), np.float32)
+    xv, mv = dev(ctx, x), dev(ctx, mask)
+    y = layer.pass_(xv, mv)
+    prog = S.Program(ctx, [y])
+    close(prog.run()[0].numpy(), torch_bert_layer(x, mask, p, heads, "gelu", 1e-12), REL_GEMM, "before")
+    loss = y.square().sum([0, 1, 2], False)
+    grads = dict(zip(layer.params(), grad(loss, layer.params())))
+    optim.Sgd(0.05).update(grads, ctx)
+    keys = ["wk", "bk", "wq", "bq", "wv", "bv", "wo", "bo", "ln1_g", "ln1_b", "w1", "b1", "w2", "b2", "ln2_g", "ln2_b"]
+    p2 = {k: v.value.numpy() for k, v in zip(keys, layer.params())}
+    assert not np.array_equal(p2["wq"], p["wq"])
+    want = torch_bert_layer(x, mask, p2, heads, "gelu", 1e-12)
+    close(prog.run()[0].numpy(), want, REL_GEMM, "replayed Program after the update")
+    close(layer.pass_(xv, mv).eval(ctx).numpy(), want, REL_GEMM, "fresh evaluation after the update")
+    prog.capture()
+    layer.params()[2].value.copy_from_numpy(p["wq"])  # host write into the query weights
+    p2["wq"] = p["wq"]
+    close(prog.run()[0].numpy(), torch_bert_layer(x, mask, p2, heads, "gelu", 1e-12), REL_GEMM, "graph replay after a host write")
+    prog.release_graph()

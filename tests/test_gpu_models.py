@@ -230,3 +230,62 @@ def test_program_graph_replay(ctx, model):
                 exact(prog.run_eager()[0].numpy(), eager[0], "eager between replays")
     finally:
         prog.release_graph()
+
+
+def test_memory_capped_evaluation_evicts_and_recomputes(ctx):
+    """Program::exec under a memory cap (session.rs:259-325): the same BERT layers evaluated in a context whose
+    capacity is a fraction of what the uncapped run holds at its peak.  Intermediates are dropped after their last
+    use, and when an allocation still does not fit, retained tensors are evicted and recomputed on demand; the
+    result is bit-identical and the allocator never hands out more than the cap."""
+    say("capped evaluation")
+    rng = np.random.default_rng(21)
+    n, l, e, heads, hdim, nlayers = 4, 128, 256, 4, 384, 8
+    layers_p = [bert_layer_params(rng, e, hdim, per_feature=True) for _ in range(nlayers)]
+    x = rng.standard_normal((n, l, e)).astype(np.float32)
+    mask = np.ones((n, l), np.float32)
+
+    def run(c):
+        h = S.Var.new(S.Tensor.from_numpy(c, x))
+        m = S.Var.new(S.Tensor.from_numpy(c, mask))
+        outs = []
+        for p in layers_p:
+            layer = BertLayer(BertConfig(e, 100, 512, hdim, 1, heads, 1e-12, 0.1, 2), reference_exact=False)
+            load_params(c, layer, layer_param_list(p))
+            h = layer.pass_(h, m)
+            outs.append(h)
+        # every layer's output has a late consumer: each must survive until then or be recomputed
+        y = outs[-1]
+        for o in outs[:-1]:
+            y = y + o
+        ev = V._Evaluator(c, [y])
+        out = ev.get(y).numpy()
+        return out, ev.evictions, c.mem_stats()
+
+    fresh = S.Context(0)
+    try:
+        want, ev0, st0 = run(fresh)
+    finally:
+        fresh.close()
+    assert ev0 == 0
+    params_bytes = sum(a.nbytes for p in layers_p for a in p.values()) + x.nbytes + mask.nbytes
+    act_peak = st0["peak"] - params_bytes  # what the uncapped run held besides parameters and inputs
+    say("uncapped peak beyond parameters", act_peak, "bytes =", act_peak / (n * l * e * 4), "activations")
+    results = []
+    for frac in (0.8, 0.7, 0.6):
+        cap = params_bytes + int(frac * act_peak)
+        c = S.Context(0, capacity=cap)
+        try:
+            got, evictions, st = run(c)
+        finally:
+            c.close()
+        exact(got, want, f"cap at {frac} of the uncapped peak")
+        assert st["peak"] <= cap, (st, cap)
+        say("cap", frac, "evictions", evictions, "peak", st["peak"])
+        results.append(evictions)
+    assert results[-1] > 0, "the tightest cap must have forced evictions"
+    hopeless = S.Context(0, capacity=params_bytes + n * l * e * 4)
+    try:
+        with pytest.raises(S.abi.OutOfMemory):
+            run(hopeless)
+    finally:
+        hopeless.close()

@@ -13,7 +13,8 @@
  *
  * What pins these restatements (see tests/test_oracle_*.py):
  *   - every tensor literal the reference's own unit tests hold (tests/golden/reference_literals.json)
- *   - closed forms in float64 (numpy/scipy) for maps, reductions, GEMM, im2col (torch unfold)
+ *   - closed forms in float64 (numpy/scipy) for maps, reductions, GEMM, im2col (torch unfold);
+ *     for col2im the adjoint identity <im2col(x), c> = <x, col2im(c)>
  *   - brute-force nested-loop index checks for translate_id / gather / scatter / slice windows.
  * Parity unpinned at ULP level: the reference evaluates exp/log/erf/pow/... and decides fma
  * contraction inside its vendor OpenCL driver, which is not part of the reference tree; these

@@ -36,8 +36,14 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));  // native vector: stays in registers
 
 constexpr int BK = 16;   // k-slab
-constexpr int KPAD = 4;  // row padding of [row][k] LDS tiles (floats)
-constexpr int RPAD = 4;  // row padding of [k][row] LDS tiles (floats)
+#ifndef SG_KPAD
+#define SG_KPAD 4
+#endif
+#ifndef SG_RPAD
+#define SG_RPAD 4
+#endif
+constexpr int KPAD = SG_KPAD;  // row padding of [row][k] LDS tiles (floats)
+constexpr int RPAD = SG_RPAD;  // row padding of [k][row] LDS tiles (floats)
 constexpr int NTHREADS = 256;
 constexpr int NUM_XCD = 8;
 
@@ -93,14 +99,24 @@ template <int ROWS, bool K_CONTIG> struct Tile {
     }
     __device__ static __forceinline__ int lds_at(int row, int k) { return K_CONTIG ? row * LD + k : k * LD + row; }
 
-    // One 16-byte item of the slab (slot i of this thread), unguarded: the whole tile lies inside
-    // the matrix and is 16-byte aligned.
-    __device__ static __forceinline__ void load_one_fast(f32x4 &r, int i, const float *base, int row0, int k0, int64_t s_row, int64_t s_k, int tid) {
+    // Unguarded loads (whole tile inside the matrix, 16-byte aligned) address an item as
+    //   uniform tile/slab base (scalar registers)  +  a per-lane 32-bit byte offset fixed for the kernel,
+    // so the K loop spends no vector instructions on addresses: lane_offset() is computed once per
+    // item before the loop, slab_base() is scalar arithmetic per slab.
+    __device__ static __forceinline__ uint32_t lane_offset(int i, uint32_t s_row, uint32_t s_k, int tid) {
         const int f = slot(tid + i * NTHREADS);
         int row, k;
         where(f, row, k);
-        const float *p = K_CONTIG ? base + (int64_t)(row0 + row) * s_row + (k0 + k) : base + (int64_t)(k0 + k) * s_k + (row0 + row);
-        r = *reinterpret_cast<const f32x4 *>(p);
+        return (K_CONTIG ? (uint32_t)row * s_row + (uint32_t)k : (uint32_t)k * s_k + (uint32_t)row) * 4u;
+    }
+    __device__ static __forceinline__ const char *tile_base(const float *base, int row0, int64_t s_row) {
+        return reinterpret_cast<const char *>(K_CONTIG ? base + (int64_t)row0 * s_row : base + row0);
+    }
+    __device__ static __forceinline__ const char *slab_base(const char *tile, int k0, int64_t s_k) {
+        return tile + (K_CONTIG ? (int64_t)k0 : (int64_t)k0 * s_k) * 4;
+    }
+    __device__ static __forceinline__ void load_one_fast(f32x4 &r, const char *slab, uint32_t lane_off) {
+        r = *reinterpret_cast<const f32x4 *>(slab + lane_off);
     }
 
     // guarded: zero-fill outside [row_lim) x [k_lim), scalar loads when 16-byte loads are not legal
@@ -220,17 +236,25 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     const int a_col = wm * WM + (lane & 31), b_col = wn * WN + (lane & 31), khalf = lane >> 5;
     float a0[TM][4], b0[TN][4], a1[TM][4], b1[TN][4];
 
+    // unguarded path: per-lane byte offsets of this thread's items inside a slab, and the tile bases
+    uint32_t off_a[TA::NV], off_b[TB::NV];
+#pragma unroll
+    for (int i = 0; i < TA::NV; ++i) off_a[i] = TA::lane_offset(i, (uint32_t)p.a_sm, (uint32_t)p.a_sk, tid);
+#pragma unroll
+    for (int i = 0; i < TB::NV; ++i) off_b[i] = TB::lane_offset(i, (uint32_t)p.b_sn, (uint32_t)p.b_sk, tid);
+    const char *a_tile = TA::tile_base(A, m0, p.a_sm), *b_tile = TB::tile_base(B, n0, p.b_sn);
+
     // item e of a slab: global memory -> registers
 #define SG_ITEM_LOAD(e, RA, RB, k0)                                                            \
     do {                                                                                       \
         if ((e) < TA::NV) {                                                                    \
             const int ia = (e) < TA::NV ? (e) : 0;                                         \
             if (GUARD) TA::load_one_guarded(RA[ia], ia, A, m0, (k0), p.M, Kloc, p.a_sm, p.a_sk, p.vec_a, tid); \
-            else TA::load_one_fast(RA[ia], ia, A, m0, (k0), p.a_sm, p.a_sk, tid);             \
+            else TA::load_one_fast(RA[ia], TA::slab_base(a_tile, (k0), p.a_sk), off_a[ia]);    \
         } else {                                                                               \
             const int ib = (e) >= TA::NV ? (e) - TA::NV : 0;                               \
             if (GUARD) TB::load_one_guarded(RB[ib], ib, B, n0, (k0), p.N, Kloc, p.b_sn, p.b_sk, p.vec_b, tid); \
-            else TB::load_one_fast(RB[ib], ib, B, n0, (k0), p.b_sn, p.b_sk, tid);             \
+            else TB::load_one_fast(RB[ib], TB::slab_base(b_tile, (k0), p.b_sk), off_b[ib]);    \
         }                                                                                      \
     } while (0)
     // item e of a slab: registers -> LDS buffer BUF
@@ -279,7 +303,15 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     // wrote before that same barrier; the g0 reads see what this iteration wrote before its barrier.
     static_assert(BK == 16, "the pipeline below is written for two groups of four k-steps per slab");
     constexpr int ITEMS3 = 2 * NWR + NRB;
-    constexpr int IPS3 = (ITEMS3 + NMFMA - 2) / (NMFMA - 1);  // items behind each MFMA of S3, last one free
+    // Which MFMA of S3 an item is issued behind: LDS writes one per MFMA from the first, then LDS reads
+    // two per MFMA, then global requests two per MFMA; the remaining MFMAs of the group run with the
+    // LDS queue draining.  (Measured against the other groupings and orders on the BERT and 4096^3
+    // shapes: coarser groups starve the matrix pipe while a wavefront issues memory instructions, finer
+    // ones for reads and requests were slower too.)
+    constexpr int W_PER = 1, R_PER = 2, G_PER = 2;
+    constexpr int SW = (NWR + W_PER - 1) / W_PER, SR = (NRB + R_PER - 1) / R_PER;
+    static_assert(SW + SR + (NWR + G_PER - 1) / G_PER <= NMFMA, "more memory items than MFMA slots in a group");
+    auto slot3 = [](int e) constexpr { return e < NWR ? e / W_PER : e < NWR + NRB ? SW + (e - NWR) / R_PER : SW + SR + (e - NWR - NRB) / G_PER; };
     constexpr int IPS5 = (NRB + NMFMA - 2) / (NMFMA - 1);
     // The body is unconditional: past the end of K the write goes to a buffer nobody reads again
     // and the fetch re-reads the last slab (unguarded path) or returns zeros (guarded path).  The
@@ -294,10 +326,11 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
         _Pragma("unroll") for (int t = 0; t < NMFMA; ++t) {                                    \
             SG_MFMA(t, a0, b0);                                                                \
             __builtin_amdgcn_sched_barrier(0);                                                 \
-            _Pragma("unroll") for (int e = t * IPS3; e < (t + 1) * IPS3; ++e) {                \
+            _Pragma("unroll") for (int e = 0; e < ITEMS3; ++e) {                               \
+                if (slot3(e) != t) continue;                                                   \
                 if (e < NWR) SG_ITEM_STORE(e, RA, RB, cur ^ 1);                                \
                 else if (e < NWR + NRB) SG_ITEM_FETCH(e - NWR, cur, 1, a1, b1);                \
-                else if (e < ITEMS3) SG_ITEM_LOAD(e - NWR - NRB, RA, RB, k_next);              \
+                else SG_ITEM_LOAD(e - NWR - NRB, RA, RB, k_next);                              \
             }                                                                                  \
             __builtin_amdgcn_sched_barrier(0);                                                 \
         }                                                                                      \
@@ -481,8 +514,12 @@ void launch_layouts(sg_ctx *ctx, const GemmP &p, dim3 grid, bool a_kc, bool b_nc
 }
 
 // GUARD = false needs every tile to lie fully inside the matrices and 16-byte loads to be legal.
-bool needs_guard(const GemmP &p, int bm, int bn) {
-    return p.M % bm != 0 || p.N % bn != 0 || p.K % (2 * BK) != 0 || !p.vec_a || !p.vec_b;
+bool needs_guard(const GemmP &p, int bm, int bn, bool a_kc, bool b_nc) {
+    // the unguarded loads keep per-lane offsets inside a tile slab in 32 bits
+    const int64_t span_a = a_kc ? (int64_t)bm * p.a_sm + BK : (int64_t)BK * p.a_sk + bm;
+    const int64_t span_b = b_nc ? (int64_t)BK * p.b_sk + bn : (int64_t)bn * p.b_sn + BK;
+    const bool fits32 = span_a >= 0 && span_b >= 0 && span_a < (1ll << 29) && span_b < (1ll << 29);
+    return p.M % bm != 0 || p.N % bn != 0 || p.K % (2 * BK) != 0 || !p.vec_a || !p.vec_b || !fits32;
 }
 
 // How many k ranges to split into.  Splitting pays when the output has too few tiles to occupy the
@@ -531,7 +568,7 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
             q.bias = nullptr; q.res = nullptr; q.alpha = 1.0f; q.act = SG_ACT_NONE; q.act_post = SG_ACT_NONE;
             q.vec_c = p.N % 4 == 0;
             dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, (unsigned)nsplit);
-            if (needs_guard(p, BM, BN)) launch_layouts<BM, BN, WAVES_M, true>(ctx, q, grid, a_kc, b_nc);
+            if (needs_guard(p, BM, BN, a_kc, b_nc)) launch_layouts<BM, BN, WAVES_M, true>(ctx, q, grid, a_kc, b_nc);
             else launch_layouts<BM, BN, WAVES_M, false>(ctx, q, grid, a_kc, b_nc);
             SG_CHECK_LAUNCH(ctx, "gemm (split-K pass 1)");
             const bool vec = p.N % 4 == 0;
@@ -545,7 +582,7 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
         }
     }
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
-    if (needs_guard(p, BM, BN)) launch_layouts<BM, BN, WAVES_M, true>(ctx, p, grid, a_kc, b_nc);
+    if (needs_guard(p, BM, BN, a_kc, b_nc)) launch_layouts<BM, BN, WAVES_M, true>(ctx, p, grid, a_kc, b_nc);
     else launch_layouts<BM, BN, WAVES_M, false>(ctx, p, grid, a_kc, b_nc);
     SG_CHECK_LAUNCH(ctx, "gemm");
     return SG_OK;

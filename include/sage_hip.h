@@ -246,6 +246,16 @@ int sg_im2col(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, const int32
 int sg_col2im(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, const int32_t ker[2],
               const int32_t stride[2], const int32_t pad[2], const int32_t dil[2]);
 
+/* ---- random fills: ops/rand.rs ------------------------------------------------------------- */
+
+/* Uniform::compute (rand.rs:62-97): out[i] = xorshift128(seed_x + i, seed_y + i) in [0, 1).
+ * Normal::compute (rand.rs:105-146): Box-Muller on xorshift128(seed_x + 2p, seed_y) and
+ * xorshift128(seed_x + 2p + 1, seed_y) for the pair p = (out[2p], out[2p+1]).  The reference draws
+ * both seeds from the host's thread_rng per call (rand.rs:70, 113); here the caller passes them.
+ * out: dense fp32. */
+int sg_rand_uniform(sg_ctx *ctx, uint32_t seed_x, uint32_t seed_y, const sg_tensor *out);
+int sg_rand_normal(sg_ctx *ctx, uint32_t seed_x, uint32_t seed_y, const sg_tensor *out);
+
 /* ---- fused row operators: compositions of ops/nn.rs ------------------------------------------ */
 
 /* softmax over the last axis (nn.rs:42-56) of (x + addend): one pass instead of reduce(max),

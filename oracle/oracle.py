@@ -702,5 +702,19 @@ def resnet18_forward(x, p):  # ResNet::new resnet.rs:75-104 with d18
     return dense(y, p["wfc"], p["bfc"])
 
 
+def rand_uniform(extents, seed_x, seed_y):  # rand.rs:62-97
+    y = HT.empty(list(extents), FLOAT)
+    yt = y.ct()
+    lib().or_rand_uniform(C.c_uint32(seed_x), C.c_uint32(seed_y), C.byref(yt))
+    return y
+
+
+def rand_normal(extents, seed_x, seed_y):  # rand.rs:105-146
+    y = HT.empty(list(extents), FLOAT)
+    yt = y.ct()
+    lib().or_rand_normal(C.c_uint32(seed_x), C.c_uint32(seed_y), C.byref(yt))
+    return y
+
+
 def num_threads():
     return lib().or_num_threads()

@@ -700,6 +700,38 @@ int or_col2im(const sg_tensor *x, const sg_tensor *out, const int32_t ker[2], co
     return OR_OK;
 }
 
+/* ---------------------------------------------------------------------------------------------
+ * Uniform::compute / Normal::compute (rand.rs:39-49, 77-83, 120-136) for given seeds.  The odd
+ * trailing element of the normal fill is the cosine branch only (the reference writes one float
+ * past its buffer there).
+ * ------------------------------------------------------------------------------------------- */
+static float or_xorshift128(uint32_t seed_x, uint32_t seed_y) {
+    const uint32_t t = seed_x ^ (seed_x << 11);
+    const uint32_t rndint = seed_y ^ (seed_y >> 19) ^ (t ^ (t >> 8));
+    return (float)rndint * 2.3283064e-10f;
+}
+
+int or_rand_uniform(uint32_t seed_x, uint32_t seed_y, const sg_tensor *out) {
+    float *y = (float *)out->base + out->offset;
+    int64_t n = numel(out);
+    for (int64_t gid = 0; gid < n; ++gid) y[gid] = or_xorshift128(seed_x + (uint32_t)gid, seed_y + (uint32_t)gid);
+    return OR_OK;
+}
+
+int or_rand_normal(uint32_t seed_x, uint32_t seed_y, const sg_tensor *out) {
+    float *y = (float *)out->base + out->offset;
+    int64_t n = numel(out);
+    for (int64_t gid = 0; 2 * gid < n; ++gid) {
+        const float u1 = or_xorshift128(seed_x + (uint32_t)gid * 2u, seed_y);
+        const float u2 = or_xorshift128(seed_x + (uint32_t)gid * 2u + 1u, seed_y);
+        const float rsq = -2.0f * logf(u1);
+        const float theta = 2.0f * 3.14159265358979323846f * u2;
+        y[2 * gid] = sqrtf(rsq) * cosf(theta);
+        if (2 * gid + 1 < n) y[2 * gid + 1] = sqrtf(rsq) * sinf(theta);
+    }
+    return OR_OK;
+}
+
 int or_num_threads(void) {
 #ifdef _OPENMP
     extern int omp_get_max_threads(void);

@@ -93,6 +93,8 @@ PROTOTYPES = {
     "sg_graph_end": (C.c_int, [_CTX, C.POINTER(C.c_void_p)]),
     "sg_graph_launch": (C.c_int, [_CTX, C.c_void_p]),
     "sg_graph_destroy": (C.c_int, [_CTX, C.c_void_p]),
+    "sg_rand_uniform": (C.c_int, [_CTX, C.c_uint32, C.c_uint32, _TP]),
+    "sg_rand_normal": (C.c_int, [_CTX, C.c_uint32, C.c_uint32, _TP]),
     "sg_attention": (C.c_int, [_CTX, _TP, _TP, _TP, _TP, C.c_float, _TP]),
 }
 

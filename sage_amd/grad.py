@@ -145,7 +145,7 @@ def _through_composition(v, gy, composed):
 def op_grad(v, gy):
     """Operation::grad (ops.rs:326-336): one entry (a Var or None) per input of `v`."""
     op, x, a = v.op, v.inputs, v.attrs
-    if op in ("literal", "data"):
+    if op in ("literal", "data", "rand_uniform", "rand_normal"):  # nullary (rand.rs:59, 102)
         return []
     if op == "unary":
         return [_unary(a["name"], x[0], v, gy)]

@@ -535,6 +535,22 @@ def matmul_batched_composed(x1, x2):
         _FUSION["on"] = on
 
 
+# ----------------------------------------------------------------------------- random fills (ops/rand.rs)
+def uniform(extents, seed=None):
+    """rand.rs:20-28.  The reference draws two 32-bit seeds from the host RNG at every evaluation
+    (rand.rs:70); `seed=(x, y)` fixes them, None draws them when the node is evaluated."""
+    if isinstance(extents, int):
+        extents = [extents]
+    return Var(Shape(list(extents)), FLOAT, "rand_uniform", attrs={"seed": tuple(seed) if seed is not None else None})
+
+
+def normal(extents, seed=None):
+    """rand.rs:30-37 (Box-Muller on xorshift128 samples)."""
+    if isinstance(extents, int):
+        extents = [extents]
+    return Var(Shape(list(extents)), FLOAT, "rand_normal", attrs={"seed": tuple(seed) if seed is not None else None})
+
+
 # ----------------------------------------------------------------------------- conv (ops/conv.rs)
 def _pair(v):
     return [int(v), int(v)] if isinstance(v, (int, np.integer)) else [int(v[0]), int(v[1])]
@@ -1055,6 +1071,18 @@ class _Evaluator:
         xc, yc = x.c(), y.c()
         self.call(self.lib.sg_im2col, C.byref(xc), C.byref(yc), arr(a["ker"]), arr(a["stride"]), arr(a["pad"]), arr(a["dil"]))
         return y
+
+    def _ev_rand(self, v):
+        seed = v.attrs["seed"]
+        if seed is None:
+            seed = tuple(int(b) for b in np.frombuffer(os.urandom(8), np.uint32))
+        y = self.out(v.extents, FLOAT)
+        yc = y.c()
+        fn = self.lib.sg_rand_uniform if v.op == "rand_uniform" else self.lib.sg_rand_normal
+        self.call(fn, C.c_uint32(seed[0] & 0xFFFFFFFF), C.c_uint32(seed[1] & 0xFFFFFFFF), C.byref(yc))
+        return y
+
+    _ev_rand_uniform = _ev_rand_normal = _ev_rand
 
     def _ev_col2im(self, v):
         x = self.get(v.inputs[0])

@@ -277,7 +277,9 @@ extern "C" int sg_im2col(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, 
     if (x->rank != 4 || out->rank != 6) return sg_fail(ctx, SG_ERR_SHAPE, "sg_im2col: x must be [N,H,W,C], out [N,OH,OW,KH,KW,C] (conv.rs:199)");
     if (!sg_is_dense(x) || !sg_is_dense(out)) return sg_fail(ctx, SG_ERR_SHAPE, "sg_im2col: x and out must be dense (conv.rs:200)");
     for (int i = 0; i < 2; ++i)
-        if (ker[i] < 1 || stride[i] < 1 || pad[i] < 0 || dil[i] < 1) return sg_fail(ctx, SG_ERR_ARG, "sg_im2col: bad geometry");
+        // dilation 0 is accepted: every tap then reads the same pixel, which is what the reference computes
+        // (its MobileNetV2 builds such convolutions, mobilenet.rs:113)
+        if (ker[i] < 1 || stride[i] < 1 || pad[i] < 0 || dil[i] < 0) return sg_fail(ctx, SG_ERR_ARG, "sg_im2col: bad geometry");
     Im2colP p;
     p.batch = (int)x->extents[0]; p.img_h = (int)x->extents[1]; p.img_w = (int)x->extents[2]; p.chan = (int)x->extents[3];
     p.ker_w = ker[0]; p.ker_h = ker[1]; p.stride_w = stride[0]; p.stride_h = stride[1];
@@ -315,6 +317,7 @@ extern "C" int sg_col2im(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, 
     if (x->rank != 6 || out->rank != 4) return sg_fail(ctx, SG_ERR_SHAPE, "sg_col2im: x must be [N,OH,OW,KH,KW,C], out [N,H,W,C] (conv.rs:243)");
     if (!sg_is_dense(x) || !sg_is_dense(out)) return sg_fail(ctx, SG_ERR_SHAPE, "sg_col2im: x and out must be dense (conv.rs:244)");
     for (int i = 0; i < 2; ++i)
+        // dilation 0 would divide by zero in the reference's kernel (conv.rs:463-465): refused
         if (ker[i] < 1 || stride[i] < 1 || pad[i] < 0 || dil[i] < 1) return sg_fail(ctx, SG_ERR_ARG, "sg_col2im: bad geometry");
     Im2colP p;
     p.batch = (int)out->extents[0]; p.img_h = (int)out->extents[1]; p.img_w = (int)out->extents[2]; p.chan = (int)out->extents[3];

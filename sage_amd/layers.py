@@ -12,9 +12,34 @@ from .tensor import FLOAT, Tensor
 from .var import Var, _pair, avg_pool_2d, conv_2d, into_var, max_pool_2d
 
 
+def _set(ctx, var, array):
+    var.set(Tensor.from_numpy(ctx, np.asarray(array, np.float32).reshape(var.extents)))
+
+
+def kaiming_uniform(rng, extents, gain=1.0):
+    """tensor/init.rs:6-15."""
+    std = gain * np.sqrt(1.0 / fan_in_out(extents)[0])
+    a = np.sqrt(3.0) * std
+    return rng.uniform(-a, a, extents).astype(np.float32)
+
+
+def kaiming_normal(rng, extents, gain=1.0):
+    """tensor/init.rs:17-25."""
+    std = gain * np.sqrt(1.0 / fan_in_out(extents)[0])
+    return (rng.standard_normal(extents) * std).astype(np.float32)
+
+
 class Layer:
     def params(self):
         return []
+
+    def init(self, ctx, rng):
+        """Parameter::init: fill this layer's parameters.  `rng` is a numpy Generator; the reference draws
+        from the host's thread_rng, so its values are not reproducible and only the distributions are mirrored."""
+        for v in vars(self).values():
+            for l in (v if isinstance(v, (list, tuple)) else [v]):
+                if isinstance(l, Layer):
+                    l.init(ctx, rng)
 
     def pass_(self, x):
         raise NotImplementedError
@@ -42,6 +67,11 @@ class Dense(Layer):
     def params(self):
         return [self.weight, self.bias]
 
+    def init(self, ctx, rng):
+        """layers.rs:224-236."""
+        _set(ctx, self.weight, kaiming_uniform(rng, self.weight.extents))
+        _set(ctx, self.bias, np.zeros(self.bias.extents))
+
     def pass_(self, x):
         return (into_var(x).matmul(self.weight) + self.bias).name("dense")
 
@@ -58,6 +88,11 @@ class Conv2d(Layer):
     def params(self):
         return [self.weight, self.bias]
 
+    def init(self, ctx, rng):
+        """layers.rs:374-386."""
+        _set(ctx, self.weight, kaiming_normal(rng, self.weight.extents))
+        _set(ctx, self.bias, np.zeros(self.bias.extents))
+
     def pass_(self, x):
         return (conv_2d(x, self.weight, self.stride, self.padding, self.dilation) + self.bias).name("conv_2d")
 
@@ -71,6 +106,10 @@ class Embedding(Layer):
 
     def params(self):
         return [self.weight]
+
+    def init(self, ctx, rng):
+        """layers.rs:466-472: standard normal."""
+        _set(ctx, self.weight, rng.standard_normal(self.weight.extents))
 
     def pass_(self, idx):
         idx = into_var(idx)
@@ -98,6 +137,11 @@ class LayerNorm(Layer):
 
     def params(self):
         return [self.gamma, self.beta]
+
+    def init(self, ctx, rng):
+        """layers.rs:570-578: gamma = beta = 1 (also beta)."""
+        _set(ctx, self.gamma, np.ones(self.gamma.extents))
+        _set(ctx, self.beta, np.ones(self.beta.extents))
 
     def pass_(self, x):
         return nn.layer_norm(x, self.axes, self.gamma, self.beta, self.eps).name("layer_norm")
@@ -171,6 +215,32 @@ class AdaptiveAvgPool2d(Layer):
         stride = [iw // ow, ih // oh]
         ker = [iw - (ow - 1) * stride[0], ih - (oh - 1) * stride[1]]
         return avg_pool_2d(x, ker, stride, [0, 0], [1, 1]).name("adaptive_avg_pool_2d")
+
+
+class BatchNorm2d(Layer):
+    """layers.rs:479-548: scalar gamma and beta, per-channel running statistics, all initialised to one; the
+    pass normalises with the RUNNING statistics (there is no batch-statistics path in the reference)."""
+
+    def __init__(self, num_features, eps):
+        self.num_features, self.eps = num_features, float(eps)
+        self.gamma = Var.empty([1]).name("batch_norm_2d.gamma")
+        self.beta = Var.empty([1]).name("batch_norm_2d.beta")
+        self.running_mean = Var.empty([num_features]).name("batch_norm_2d.running_mean")
+        self.running_var = Var.empty([num_features]).name("batch_norm_2d.running_var")
+
+    def params(self):
+        return [self.gamma, self.beta]
+
+    def init(self, ctx, rng):
+        _set(ctx, self.gamma, np.ones(1))
+        _set(ctx, self.beta, np.ones(1))
+        _set(ctx, self.running_mean, np.ones(self.num_features))
+        _set(ctx, self.running_var, np.ones(self.num_features))
+
+    def pass_(self, x):
+        from .var import batch_norm_2d
+        # the eps given to the constructor is ignored: the pass hard-codes 1e-05 (layers.rs:541-543)
+        return batch_norm_2d(x, self.gamma, self.beta, self.running_mean, self.running_var, 1e-05).name("batch_norm_2d")
 
 
 class Sequential(Layer):

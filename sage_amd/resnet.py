@@ -19,6 +19,18 @@ class ResNetConfig:
     def d34(chan_input, num_classes):
         return ResNetConfig(chan_input, num_classes, [3, 4, 6, 3], 1, False)
 
+    @staticmethod
+    def d50(chan_input, num_classes):
+        return ResNetConfig(chan_input, num_classes, [3, 4, 6, 3], 4, True)
+
+    @staticmethod
+    def d101(chan_input, num_classes):
+        return ResNetConfig(chan_input, num_classes, [3, 4, 23, 3], 4, True)
+
+    @staticmethod
+    def d152(chan_input, num_classes):
+        return ResNetConfig(chan_input, num_classes, [3, 8, 36, 3], 4, True)
+
 
 class BasicLayer(Layer):
     """resnet.rs:155-176, 270-279."""
@@ -39,12 +51,23 @@ class BasicLayer(Layer):
         return nn.relu(y)
 
 
+class BottleneckLayer(BasicLayer):
+    """resnet.rs:178-243: 1x1 -> 3x3 (stride) -> 1x1 (expansion), same shortcut rule as the basic block."""
+
+    def __init__(self, in_planes, planes, stride, config):
+        out_planes = config.expansion * planes
+        self.main = Sequential(Conv2d(in_planes, planes, 1), Relu(), Conv2d(planes, planes, 3, stride, 1, 1), Relu(),
+                               Conv2d(planes, out_planes, 1))
+        self.downsample = None
+        if stride != 1 or in_planes != out_planes:
+            self.downsample = Sequential(Conv2d(in_planes, out_planes, 1, stride, 0, 1))
+
+
 class ResNet(Layer):
     """resnet.rs:75-130."""
 
     def __init__(self, config):
-        if config.use_bottleneck:
-            raise NotImplementedError("bottleneck variants (d50+) are outside the ResNet-18 configuration")
+        block = BottleneckLayer if config.use_bottleneck else BasicLayer
         m = Sequential()
         in_planes = 64
         out_planes = in_planes
@@ -55,7 +78,7 @@ class ResNet(Layer):
             stride = 1 if i == 0 else 2
             ip = in_planes
             for b in range(config.num_blocks[i]):
-                m.add(BasicLayer(ip, out_planes, stride if b == 0 else 1, config))
+                m.add(block(ip, out_planes, stride if b == 0 else 1, config))
                 ip = out_planes * config.expansion
             in_planes = out_planes * config.expansion
             out_planes *= 2

@@ -738,6 +738,30 @@ class Program:
         return self.outputs
 
 
+def _allow_depth(targets):
+    """The evaluator walks the graph recursively, a handful of Python frames per node: raise the
+    interpreter's recursion limit to fit the deepest chain of this graph (MobileNetV2 is ~400 nodes deep)."""
+    import sys
+    depth, memo = 0, {}
+    for t in targets:
+        stack = [t]
+        while stack:
+            n = stack[-1]
+            if id(n) in memo:
+                stack.pop()
+                continue
+            todo = [i for i in n.inputs if id(i) not in memo] if n.value is None else []
+            if todo:
+                stack.extend(todo)
+                continue
+            memo[id(n)] = 1 + max((memo[id(i)] for i in n.inputs), default=0) if n.value is None else 0
+            stack.pop()
+        depth = max(depth, memo[id(t)])
+    need = min(12 * depth + 1000, 60000)
+    if sys.getrecursionlimit() < need:
+        sys.setrecursionlimit(need)
+
+
 def _merge_common_subgraphs(targets):
     """Structurally identical operations on the same inputs are computed once: inputs of every node are
     re-pointed at the first node seen with the same (operator, attributes, inputs).  BERT rebuilds the
@@ -775,6 +799,7 @@ class _Evaluator:
         self.targets = {id(t) for t in targets}
         if _FUSION["on"]:
             _merge_common_subgraphs(targets)
+        _allow_depth(targets)
         seen = set()
         stack = list(targets)
         while stack:

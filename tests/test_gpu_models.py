@@ -289,3 +289,33 @@ def test_memory_capped_evaluation_evicts_and_recomputes(ctx):
             run(hopeless)
     finally:
         hopeless.close()
+
+
+@pytest.mark.parametrize("name", ["densenet121", "mobilenetv2", "resnet50"])
+def test_other_model_families_vs_oracle(ctx, name):
+    """DenseNet (densenet.rs), MobileNetV2 (mobilenet.rs, with its dilation-0 3x3 stage) and the bottleneck ResNets
+    (resnet.rs:178-243): parameters from the layers' own init, forward pass against the oracle's layer-by-layer
+    evaluation of the same layer tree; fused and operator-by-operator evaluation agree."""
+    from sage_amd.densenet import DenseNet, DenseNetConfig
+    from sage_amd.mobilenet import MobileNetV2, MobileNetV2Config
+    from tests import oracle_layers
+    say("model", name)
+    rng = np.random.default_rng(7)
+    model = {"densenet121": lambda: DenseNet(DenseNetConfig.d121(3, 10)), "mobilenetv2": lambda: MobileNetV2(MobileNetV2Config(3, 10)),
+             "resnet50": lambda: ResNet(ResNetConfig.d50(3, 10))}[name]()
+    model.init(ctx, rng)
+    for p in model.params():  # biases start at zero (layers.rs:233, 383): give them values so they are exercised
+        if p.rank == 1:
+            p.set(S.Tensor.from_numpy(ctx, (rng.standard_normal(p.extents) * 0.1).astype(np.float32)))
+    x = rng.uniform(0, 1, (2, 32, 32, 3)).astype(np.float32)
+    n0 = ctx.launches
+    y = model.pass_(dev(ctx, x)).eval(ctx).numpy()
+    fused = ctx.launches - n0
+    yo = oracle_layers.forward(model, ht(x)).numpy()
+    assert y.shape == (2, 10) and np.all(np.isfinite(y))
+    close(y, yo, REL_GEMM, "fused vs oracle")
+    V.set_fusion(False)
+    n0 = ctx.launches
+    y2 = model.pass_(dev(ctx, x)).eval(ctx).numpy()
+    close(y2, yo, REL_GEMM, "operator by operator vs oracle")
+    say("launches", fused, "fused,", ctx.launches - n0, "operator by operator")

@@ -254,3 +254,24 @@ def test_gradient_graph_construction():
         ops.add(v.op)
         stack.extend(v.inputs)
     assert "col2im" in ops and "gemm" in ops and "cond" in ops  # conv backward, dense backward, max-pool backward
+
+
+def test_model_families_build_without_a_device():
+    """densenet.rs, mobilenet.rs, resnet.rs (bottleneck variants): layer trees and output shapes."""
+    from sage_amd.densenet import DenseNet, DenseNetConfig
+    from sage_amd.layers import fan_in_out, kaiming_normal, kaiming_uniform
+    from sage_amd.mobilenet import MobileNetV2, MobileNetV2Config, make_divisible
+    from sage_amd.resnet import ResNet, ResNetConfig
+    from sage_amd.var import Var
+    assert [make_divisible(v, 8, 8) for v in (32, 16, 24, 1280, 3, 100)] == [32, 16, 24, 1280, 8, 104]  # mobilenet.rs:10-18
+    x = Var.empty([2, 32, 32, 3])
+    for model, nparams in ((DenseNet(DenseNetConfig.d121(3, 10)), 236), (MobileNetV2(MobileNetV2Config(3, 10)), 106),
+                           (ResNet(ResNetConfig.d50(3, 10)), 108), (ResNet(ResNetConfig.d18(3, 10)), 42)):
+        assert model.pass_(x).extents == [2, 10]
+        assert len(model.params()) == nparams
+    # tensor/init.rs:27-50: fan_in = extents[1] * prod(extents[2:])
+    assert fan_in_out([3, 3, 16, 32]) == (3 * 16 * 32, 3 * 16 * 32)
+    rng = np.random.default_rng(0)
+    w = kaiming_uniform(rng, [64, 256])
+    assert w.dtype == np.float32 and np.abs(w).max() <= np.sqrt(3.0 / 256) + 1e-7
+    assert abs(float(kaiming_normal(rng, [3, 3, 64, 64]).std()) - np.sqrt(1.0 / (3 * 64 * 64))) < 2e-3

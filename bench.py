@@ -29,13 +29,18 @@ PEAK_HBM_GBS = 8000.0
 
 def measured_traffic(kernel, workload):
     """HBM bytes per dispatch of `kernel` from the committed rocprofv3 counter summary of this same
-    workload (profiles/traffic_<workload>.json: FETCH_SIZE and WRITE_SIZE runs scaled by a copy kernel
-    of known size), or None when there is no such measurement."""
-    path = os.path.join(ROOT, "profiles", f"traffic_{workload}.json")
+    workload (FETCH_SIZE and WRITE_SIZE runs scaled by a copy kernel of known size), or None when there
+    is no such measurement.  profiles/traffic_<workload>.json holds every kernel of a model workload;
+    profiles/traffic_single_kernel_workloads.json holds the one timed kernel of each single-kernel workload."""
     try:
-        with open(path) as f:
+        with open(os.path.join(ROOT, "profiles", f"traffic_{workload}.json")) as f:
             k = json.load(f)["kernels"].get(kernel)
         return k["traffic_bytes_per_dispatch"] if k else None
+    except (OSError, ValueError, KeyError):
+        pass
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic_single_kernel_workloads.json")) as f:
+            return json.load(f)["workloads"][workload]["traffic_bytes_per_dispatch"]
     except (OSError, ValueError, KeyError):
         return None
 
@@ -236,6 +241,10 @@ def kernel_workloads(ctx, name, rng):
         nbuf = 20
         progs = programs(lambda i: dev(rng.standard_normal((B, Cn)).astype(np.float32)).sum(1, True), nbuf)
         return progs, B * Cn * 4 + B * 4, 0.0, "reduce_row_kernel", None
+    if name == "copy":            # plain copy of 64 Mi floats: the kernel of known size that calibrates FETCH_SIZE / WRITE_SIZE
+        n = 64 << 20
+        progs = programs(lambda i: dev(np.ones(n, np.float32)).copy(), 1)
+        return progs, 2 * n * 4, 0.0, "sg_map", None
     if name == "gemm_bias":       # config 2: C = A@B + bias, 4096^3
         M = N = K = 4096
         A, Bm, bias = (dev(rng.uniform(-1, 1, s).astype(np.float32)) for s in ((M, K), (K, N), (N,)))
@@ -311,8 +320,8 @@ def run_kernel_workload(a):
            "data": "synthetic",
            "config": {"workload": a.workload, "launches_per_step": launches, "buffer_sets": len(progs),
                       "algorithmic_bytes_per_step": bytes_per, "flops_per_step": flops_per},
-           "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak, "traffic": None,
-                        "kernel": label, "avg_launch_ms": per_ms}}
+           "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
+                        "traffic": measured_traffic(label, a.workload), "kernel": label, "avg_launch_ms": per_ms}}
     if spec is not None and not a.no_cpu_baseline:
         t, sample = oracle_kernel_baseline(spec, np.random.default_rng(2))
         if t:
@@ -374,7 +383,7 @@ def run_train_workload(a):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="bert", help="bert (default, the headline metric) | resnet18 | resnet18_train | softmax_ce | map_exp_sub | "
+    ap.add_argument("--workload", default="bert", help="bert (default, the headline metric) | resnet18 | resnet18_train | copy | softmax_ce | map_exp_sub | "
                     "bias_residual | layer_norm | softmax | reduce_sum | gemm_bias")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)

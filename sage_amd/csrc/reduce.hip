@@ -130,8 +130,18 @@ __global__ void __launch_bounds__(256) reduce_row_kernel(const T *__restrict__ x
         if (VEC4) {
             typedef T V4 __attribute__((ext_vector_type(4)));
             const V4 *p4 = reinterpret_cast<const V4 *>(p);
-            for (uint32_t i = t; i < len / 4; i += nt) {
-                V4 v = p4[i];
+            // four loads in flight per trip; the values are combined in the order a one-load loop would
+            const uint32_t n4 = len / 4;
+            uint32_t i = t;
+            for (; i + 3 * nt < n4; i += 4 * nt) {
+                const V4 v0 = p4[i], v1 = p4[i + nt], v2 = p4[i + 2 * nt], v3 = p4[i + 3 * nt];
+                acc = combine<OP, T>(combine<OP, T>(combine<OP, T>(combine<OP, T>(acc, v0.x), v0.y), v0.z), v0.w);
+                acc = combine<OP, T>(combine<OP, T>(combine<OP, T>(combine<OP, T>(acc, v1.x), v1.y), v1.z), v1.w);
+                acc = combine<OP, T>(combine<OP, T>(combine<OP, T>(combine<OP, T>(acc, v2.x), v2.y), v2.z), v2.w);
+                acc = combine<OP, T>(combine<OP, T>(combine<OP, T>(combine<OP, T>(acc, v3.x), v3.y), v3.z), v3.w);
+            }
+            for (; i < n4; i += nt) {
+                const V4 v = p4[i];
                 acc = combine<OP, T>(combine<OP, T>(combine<OP, T>(combine<OP, T>(acc, v.x), v.y), v.z), v.w);
             }
         } else {
@@ -218,6 +228,10 @@ __global__ void __launch_bounds__(256) reduce_arg_row_kernel(const T *__restrict
 // lane; short rows use a fraction of it, so one wavefront carries 64/LPR rows and every load
 // instruction still moves 1 KiB.  Reductions run over the LPR lanes of a row with xor shuffles.
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// e^t through the hardware 2^x: relative error about |t| * 6e-8 from the rounded argument plus one ulp;
+// results below 2^-126 come out as zero.
+__device__ __forceinline__ float fast_exp(float t) { return __builtin_amdgcn_exp2f(t * 1.44269504088896340736f); }
 
 template <int NCHUNK> struct RowRegs {
     f32x4 v[NCHUNK];
@@ -335,21 +349,40 @@ __global__ void __launch_bounds__(256) softmax_ce_row_kernel(const float *__rest
     const uint32_t row = (blockIdx.x * 4u + wave) * RPW + lane / LPR;
     if (row >= n_rows) return;
     const float *p = x + x_off + (size_t)row * x_row_stride;
+    // the label is requested with the row, and x[label] is then picked out of the row's registers: no
+    // dependent load waits at the end of the wavefront's life
+    const uint32_t label = labels[l_off + (size_t)row * l_stride];
     RowRegs<NCHUNK> r;
     load_row<NCHUNK, LPR>(p, len, li, r, -__builtin_inff());
+    float picked = 0.0f;  // x[label] on the lane that holds it (a label outside the row leaves 0 on every lane)
+#pragma unroll
+    for (int j = 0; j < NCHUNK; ++j) {
+        const uint32_t c = (j * LPR + li) * 4u;
+        if (label - c < 4u) picked = r.v[j][label - c];
+    }
     float m = -__builtin_inff();
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) m = fmaxf(fmaxf(fmaxf(fmaxf(m, r.v[j].x), r.v[j].y), r.v[j].z), r.v[j].w);
     m = fmaxf(seg_reduce<OP_MAX, LPR>(m), 0.0f);  // the reference's max accumulator starts at 0 (reduce.rs:282)
+    const float xl = seg_reduce<OP_SUM, LPR>(picked);  // one lane holds the value, the others 0: the sum is exact
     float s = 0.0f;
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j)
-        s += (expf(r.v[j].x - m) + expf(r.v[j].y - m)) + (expf(r.v[j].z - m) + expf(r.v[j].w - m));
+        s += (fast_exp(r.v[j].x - m) + fast_exp(r.v[j].y - m)) + (fast_exp(r.v[j].z - m) + fast_exp(r.v[j].w - m));
     s = seg_reduce<OP_SUM, LPR>(s);
+    // fast_exp flushes results below 2^-126 to zero.  They only matter to the sum when every term is
+    // that small (a row entirely below -87): then the sum is redone with the exact routine, which
+    // keeps the denormal terms as the reference's kernel language does.
+    if (s < 1.0e-30f) {
+        s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NCHUNK; ++j)
+            s += (expf(r.v[j].x - m) + expf(r.v[j].y - m)) + (expf(r.v[j].z - m) + expf(r.v[j].w - m));
+        s = seg_reduce<OP_SUM, LPR>(s);
+    }
     if (li == 0) {
-        const uint32_t label = labels[l_off + (size_t)row * l_stride];
         const float lse = logf(s) + m;
-        loss[y_off + row] = -(p[label] - lse);
+        loss[y_off + row] = -(xl - lse);
     }
 }
 
@@ -397,6 +430,26 @@ __global__ void __launch_bounds__(256) layer_norm_row_kernel(const float *__rest
     const float *p = x + x_off + decompose(xo, row);
     RowRegs<NCHUNK> r;
     load_row<NCHUNK, LPR>(p, len, li, r, 0.0f);
+    // gamma and beta are requested with the row, so nothing waits on memory after the statistics
+    const bool vec_params = g_stride == 1 && b_stride == 1 && ((g_off | b_off) & 3u) == 0;
+    f32x4 gv[NCHUNK], bv[NCHUNK];
+#pragma unroll
+    for (int j = 0; j < NCHUNK; ++j) {
+        const uint32_t c = (j * LPR + li) * 4u;
+        gv[j] = bv[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (c < len) {
+            if (vec_params) {
+                gv[j] = *reinterpret_cast<const f32x4 *>(gamma + g_off + c);
+                bv[j] = *reinterpret_cast<const f32x4 *>(beta + b_off + c);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    gv[j][t] = gamma[g_off + (c + t) * g_stride];
+                    bv[j][t] = beta[b_off + (c + t) * b_stride];
+                }
+            }
+        }
+    }
     float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
@@ -410,24 +463,10 @@ __global__ void __launch_bounds__(256) layer_norm_row_kernel(const float *__rest
     const float var = s2 / n - mean * mean;
     const float inv = 1.0f / sqrtf(var + eps);
     float *q = y + y_off + (size_t)row * len;
-    const bool vec_params = g_stride == 1 && b_stride == 1 && ((g_off | b_off) & 3u) == 0;
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
-        uint32_t c = (j * LPR + li) * 4u;
-        if (c < len) {
-            f32x4 g, b;
-            if (vec_params) {
-                g = *reinterpret_cast<const f32x4 *>(gamma + g_off + c);
-                b = *reinterpret_cast<const f32x4 *>(beta + b_off + c);
-            } else {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    g[t] = gamma[g_off + (c + t) * g_stride];
-                    b[t] = beta[b_off + (c + t) * b_stride];
-                }
-            }
-            *reinterpret_cast<f32x4 *>(q + c) = (r.v[j] - mean) * inv * g + b;
-        }
+        const uint32_t c = (j * LPR + li) * 4u;
+        if (c < len) *reinterpret_cast<f32x4 *>(q + c) = (r.v[j] - mean) * inv * gv[j] + bv[j];
     }
 }
 
@@ -570,16 +609,17 @@ int64_t row_dims(const sg_tensor *t, Dims &d) {
 
 }  // namespace
 
-// Rows of up to 256 floats are dealt to 4..64 lanes (one chunk each, several rows per wavefront);
-// longer rows to all 64 lanes with 2..8 chunks per lane.  Expects SG_ROW_LAUNCH(NCHUNK, LPR).
+// Rows of up to 64 floats are dealt to 4..16 lanes (one 16-byte chunk each), rows of up to 256 to 8 or 16
+// lanes with four chunks each (several rows per wavefront, 64 bytes in flight per lane: measured faster
+// than one chunk on 32 or 64 lanes); longer rows to all 64 lanes with 2..8 chunks per lane.  Expects SG_ROW_LAUNCH(NCHUNK, LPR).
 #define SG_ROW_DISPATCH(LEN)                                                                                            \
     do {                                                                                                                \
         const uint32_t len_ = (LEN);                                                                                    \
         if (len_ <= 16) SG_ROW_LAUNCH(1, 4);                                                                            \
         else if (len_ <= 32) SG_ROW_LAUNCH(1, 8);                                                                       \
         else if (len_ <= 64) SG_ROW_LAUNCH(1, 16);                                                                      \
-        else if (len_ <= 128) SG_ROW_LAUNCH(1, 32);                                                                     \
-        else if (len_ <= 256) SG_ROW_LAUNCH(1, 64);                                                                     \
+        else if (len_ <= 128) SG_ROW_LAUNCH(4, 8);                                                                      \
+        else if (len_ <= 256) SG_ROW_LAUNCH(4, 16);                                                                     \
         else if (len_ <= 512) SG_ROW_LAUNCH(2, 64);                                                                     \
         else if (len_ <= 768) SG_ROW_LAUNCH(3, 64);                                                                     \
         else if (len_ <= 1024) SG_ROW_LAUNCH(4, 64);                                                                    \

@@ -5,6 +5,7 @@
 // accounting of Pool::alloc / check_space (session/memory.rs:246-255, 353-362).
 #include "common.h"
 
+#include <cstdlib>
 #include <cstring>
 
 int sg_fail(sg_ctx *ctx, int code, const char *fmt, ...) {
@@ -17,6 +18,14 @@ int sg_fail(sg_ctx *ctx, int code, const char *fmt, ...) {
         ctx->last_error = buf;
     }
     return code;
+}
+
+bool sg_streaming(int64_t bytes) {
+    static const int64_t min_bytes = [] {
+        const char *e = getenv("SAGE_STREAM_MIN_BYTES");
+        return e ? (int64_t)strtoll(e, nullptr, 10) : (int64_t)32 << 20;
+    }();
+    return bytes >= min_bytes;
 }
 
 int sg_validate_tensor(sg_ctx *ctx, const sg_tensor *t, const char *name) {

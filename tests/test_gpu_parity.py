@@ -645,6 +645,28 @@ def test_softmax_cross_entropy(ctx, shape):
     close(yf, yo, REL_MAP, "fused vs oracle")
 
 
+def test_softmax_cross_entropy_rows_far_below_zero(ctx):
+    """The shift is max(0, row max) (reduce.rs:282), so a row entirely below -87 sums terms under 2^-126:
+    the fused kernel keeps them (denormal) like the composition and the oracle, it does not flush the sum
+    to zero and the loss to infinity.  Rows partly below that limit and ordinary rows ride along."""
+    say("softmax_cross_entropy far below zero")
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((64, 1024)).astype(np.float32)
+    x[:16] = rng.uniform(-101.0, -89.0, (16, 1024)).astype(np.float32)     # every term denormal
+    x[16:32] = rng.uniform(-95.0, -80.0, (16, 1024)).astype(np.float32)    # denormal and normal terms mixed
+    x[32:40] -= 60.0
+    lab = rng.integers(0, 1024, (64, 1)).astype(np.int32)
+    yf = nn.softmax_cross_entropy(dev(ctx, x), dev(ctx, lab)).eval(ctx).numpy()
+    yo = O.softmax_cross_entropy(ht(x), ht(lab.view(np.uint32))).numpy()
+    assert np.all(np.isfinite(yo)) and np.all(np.isfinite(yf))
+    x64 = x.astype(np.float64)
+    ref = -(x64[np.arange(64), lab[:, 0]] - np.log(np.exp(x64).sum(1)))
+    # denormal terms carry fewer bits: the all-denormal rows agree to 1e-2 absolute on losses near 10, the rest to REL_MAP
+    assert np.max(np.abs(yf[:16] - yo[:16])) < 1e-2 and np.max(np.abs(yf[:16] - ref[:16])) < 0.1
+    close(yf[16:], yo[16:], REL_MAP, "fused vs oracle")
+    close(yf[16:], ref[16:], REL_MAP, "fused vs float64")
+
+
 @pytest.mark.parametrize("shape,per_feature", [((8, 16, 768), False), ((8, 16, 768), True), ((5, 100), False), ((3, 2050), True), ((64, 64), True)])
 def test_layer_norm(ctx, shape, per_feature):
     say("layer_norm", shape, per_feature)

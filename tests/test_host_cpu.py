@@ -162,13 +162,18 @@ COND = (abi.EXPR_TERNARY, 0, 0, 0)
 
 
 def test_map_source_vector_path_and_compile():
-    """exp(x0 - x1), x1 broadcast per row: 16-byte loads for x0, one scalar load for x1."""
+    """exp(x0 - x1), x1 broadcast per row: 16-byte loads for x0, one scalar load for x1; 67 MB of operands
+    are streamed (non-temporal), a small map of the same expression is not."""
     x0 = desc([8192, 1024])
     x1 = desc([8192, 1024], [1, 0])
     rc, src, dt = source([UN("exp"), BIN("sub"), INP(0), INP(1)], [x0, x1], desc([8192, 1024]))
     assert rc == abi.OK and dt == abi.FLOAT
-    assert "const float4 v0" in src and "const float s1" in src and "expf((x0 - x1))" in src
+    assert "const sg_float4 v0 = __builtin_nontemporal_load(" in src and "const float s1" in src and "expf((x0 - x1))" in src
+    assert "__builtin_nontemporal_store(r," in src
     compiles(src)
+    rc, small, _ = source([UN("exp"), BIN("sub"), INP(0), INP(1)], [desc([64, 1024]), desc([64, 1024], [1, 0])], desc([64, 1024]))
+    assert rc == abi.OK and "const sg_float4 v0 = *(" in small and "nontemporal" not in small.split("extern")[1]
+    compiles(small)
 
 
 def test_map_source_scalar_path_for_transposed_operand():
@@ -183,7 +188,7 @@ def test_map_source_collapses_dense_axes():
     assert rc == abi.OK and "#define ND 1" in src
     bias = desc([32, 128, 768], [0, 0, 1])
     rc, src, _ = source([BIN("add"), INP(0), INP(1)], [desc([32, 128, 768]), bias], desc([32, 128, 768]))
-    assert rc == abi.OK and "#define ND 2" in src and "const float4 v1" in src
+    assert rc == abi.OK and "#define ND 2" in src and "const sg_float4 v1" in src
 
 
 def test_every_map_operator_compiles_for_gfx950():

@@ -211,7 +211,7 @@ def kernel_workloads(ctx, name, rng):
         nbuf = 20
         lab = rng.integers(0, Cn, (B, 1)).astype(np.int32)
         progs = programs(lambda i: nn.softmax_cross_entropy(dev(rng.standard_normal((B, Cn)).astype(np.float32)), dev(lab)), nbuf)
-        return progs, B * Cn * 4 + B * 4 + B * 4, 0.0, "softmax_ce_row_kernel<4>", ("softmax_ce", B, Cn)
+        return progs, B * Cn * 4 + B * 4 + B * 4, 0.0, "softmax_ce_row_kernel<4, 64>", ("softmax_ce", B, Cn)
     if name == "map_exp_sub":     # exp(x0 - x1), x1 broadcast per row (the largest map of config 1)
         B, Cn = 8192, 1024
         nbuf = 12
@@ -229,18 +229,18 @@ def kernel_workloads(ctx, name, rng):
         nbuf = 6
         g, b = dev(np.ones(Cn, np.float32)), dev(np.zeros(Cn, np.float32))
         progs = programs(lambda i: nn.layer_norm(dev(rng.standard_normal((R, Cn)).astype(np.float32)), 1, g, b, 1e-12), nbuf)
-        return progs, 2 * R * Cn * 4 + 2 * Cn * 4, 0.0, "layer_norm_row_kernel<3>", None
+        return progs, 2 * R * Cn * 4 + 2 * Cn * 4, 0.0, "layer_norm_row_kernel<3, 64>", None
     if name == "softmax":         # attention scores [32,12,128,128] + mask
         n, h, l = 32, 12, 128
         nbuf = 12
         m = dev(np.zeros((n, 1, 1, l), np.float32))
         progs = programs(lambda i: nn.softmax(dev(rng.standard_normal((n, h, l, l)).astype(np.float32)) + m, 3), nbuf)
-        return progs, 2 * n * h * l * l * 4 + n * l * 4, 0.0, "softmax_row_kernel<1, true>", None
+        return progs, 2 * n * h * l * l * 4 + n * l * 4, 0.0, "softmax_row_kernel<4, 8, true>", None
     if name == "reduce_sum":      # row sums of [8192,1024]
         B, Cn = 8192, 1024
         nbuf = 20
         progs = programs(lambda i: dev(rng.standard_normal((B, Cn)).astype(np.float32)).sum(1, True), nbuf)
-        return progs, B * Cn * 4 + B * 4, 0.0, "reduce_row_kernel", None
+        return progs, B * Cn * 4 + B * 4, 0.0, "reduce_row_kernel<0, float, true, false>", None
     if name == "copy":            # plain copy of 64 Mi floats: the kernel of known size that calibrates FETCH_SIZE / WRITE_SIZE
         n = 64 << 20
         progs = programs(lambda i: dev(np.ones(n, np.float32)).copy(), 1)
@@ -386,8 +386,8 @@ def main():
     ap.add_argument("--workload", default="bert", help="bert (default, the headline metric) | resnet18 | resnet18_train | copy | softmax_ce | map_exp_sub | "
                     "bias_residual | layer_norm | softmax | reduce_sum | gemm_bias")
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default 30; 2000 for the single-kernel workloads, whose step is microseconds)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default 5; 500 for the single-kernel workloads)")
     ap.add_argument("--variant", choices=["config", "reference"], default="config")
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--seq", type=int, default=128)
@@ -396,6 +396,11 @@ def main():
     ap.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
                     help="replay the step as one HIP graph (auto: on for resnet18, whose step is bound by host launches)")
     a = ap.parse_args()
+    single_kernel = a.workload not in ("bert", "resnet18", "resnet18_train")
+    if a.steps is None:
+        a.steps = 2000 if single_kernel else 30
+    if a.warmup is None:
+        a.warmup = 500 if single_kernel else 5
     if a.gpus != 1:
         print("bench.py measures one GPU: every box in this run has one MI355X and the hot path uses no "
               "collectives; run with --gpus 1", file=sys.stderr)

@@ -149,7 +149,6 @@ template <class A, class B> __device__ __forceinline__ auto sg_max(A a, B b) -> 
 struct MapPlan {
     int ndim = 1;
     int vec = 1;
-    int unroll = 1;  // independent vectors per thread
     bool stream = false;  // operands too large to be reused from cache: non-temporal loads and stores
     uint32_t ext[SG_MAX_RANK];
     uint32_t stride[SG_MAX_MAP_INPUTS][SG_MAX_RANK];
@@ -212,9 +211,6 @@ void plan_map(const sg_tensor *in, int n_in, const sg_tensor *out, MapPlan &pl) 
     int64_t total = 1;
     for (int a = 0; a < nd; ++a) total *= ext[a];
     total /= pl.vec;
-    // one 16-byte vector per thread: measured against 2, 4 and 8 per thread and against grid-stride
-    // loops on 64 MB..512 MB copies and fused maps, the plain one-vector grid sustains the most
-    pl.unroll = 1;
     int64_t bytes = sg_numel(out) * 4;
     for (int k = 0; k < n_in; ++k) {
         int64_t distinct = 1;
@@ -241,8 +237,9 @@ std::string gen_source(const std::string &expr, const sg_tensor *in, int n_in, i
     s << "extern \"C\" __global__ void __launch_bounds__(256) sg_map(";
     for (int k = 0; k < n_in; ++k) s << "const " << ctype(in[k].dtype) << " *__restrict__ b" << k << ", ";
     s << ctype(out_dt) << " *__restrict__ yb, const MapParams p) {\n";
-    s << "  const uint base = blockIdx.x * " << 256 * pl.unroll << "u + threadIdx.x;\n";
-    s << "#pragma unroll\n  for (uint u = 0; u < " << pl.unroll << "u; ++u) {\n  const uint gid = base + u * 256u;\n  if (gid < p.total) {\n";
+    // one 16-byte vector (or one element) per thread: measured against 2, 4 and 8 vectors per thread and
+    // against grid-stride loops on 64 MB..512 MB copies and fused maps, this plain grid sustains the most
+    s << "  const uint gid = blockIdx.x * 256u + threadIdx.x;\n  if (gid < p.total) {\n";
     if (pl.need_coords) {
         // coordinates in units of V elements along the innermost axis
         s << "  uint rem = gid, q;\n";
@@ -291,7 +288,7 @@ std::string gen_source(const std::string &expr, const sg_tensor *in, int n_in, i
         if (pl.stream) s << "  __builtin_nontemporal_store(r, reinterpret_cast<sg_" << odt << "4 *>(yb + p.yoff + gid * 4u));\n";
         else s << "  *reinterpret_cast<sg_" << odt << "4 *>(yb + p.yoff + gid * 4u) = r;\n";
     }
-    s << "  }\n  }\n}\n";
+    s << "  }\n}\n";
     return s.str();
 }
 
@@ -445,8 +442,7 @@ extern "C" int sg_map(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_ten
     ptrs[n_in] = out->base;
     args.push_back(&ptrs[n_in]);
     args.push_back(params.data());
-    const int64_t per_block = 256 * pl.unroll;
-    const unsigned grid = (unsigned)((total + per_block - 1) / per_block);
+    const unsigned grid = (unsigned)((total + 255) / 256);
     SG_HIP(ctx, hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr));
     return SG_OK;
 }

@@ -30,6 +30,8 @@
 // order); the difference is fp32 rounding only and is covered by the 1e-3 GEMM tolerance.
 #include "common.h"
 
+#include <type_traits>
+
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -66,8 +68,16 @@ struct GemmP {
 
 __device__ __forceinline__ float apply_act(float v, int act) {
     if (act == SG_ACT_RELU) return v > 0.0f ? v : 0.0f * v;  // (float)(v>0) * v, nn.rs:39
-    if (act == SG_ACT_GELU_ERF) return (v * 0.5f) * (erff(v / 1.41421356237309504880f) + 1.0f);
+    if (act == SG_ACT_GELU_ERF) return (v * 0.5f) * (erff(v * 0.70710678118654752440f) + 1.0f);
     return v;
+}
+// the same for the four values of a lane, with one uniform branch on the kind instead of four
+__device__ __forceinline__ void apply_act4(f32x4 &v, int act) {
+    if (act == SG_ACT_RELU) {
+        v.x = apply_act(v.x, SG_ACT_RELU); v.y = apply_act(v.y, SG_ACT_RELU); v.z = apply_act(v.z, SG_ACT_RELU); v.w = apply_act(v.w, SG_ACT_RELU);
+    } else if (act == SG_ACT_GELU_ERF) {
+        v.x = apply_act(v.x, SG_ACT_GELU_ERF); v.y = apply_act(v.y, SG_ACT_GELU_ERF); v.z = apply_act(v.z, SG_ACT_GELU_ERF); v.w = apply_act(v.w, SG_ACT_GELU_ERF);
+    }
 }
 
 // One operand tile (ROWS x BK; rows are m or n indices) on its way from global memory to LDS.
@@ -385,7 +395,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
         const bool n_in = !GUARD || n + 3 < p.N;
         bias = f32x4{0.f, 0.f, 0.f, 0.f};
         if (p.bias) {
-            if (p.vec_bias && n_in) bias = *reinterpret_cast<const f32x4 *>(p.bias + n);
+            if (!GUARD || (p.vec_bias && n_in)) bias = *reinterpret_cast<const f32x4 *>(p.bias + n);
             else {
                 if (n + 0 < p.N) bias.x = p.bias[n + 0];
                 if (n + 1 < p.N) bias.y = p.bias[n + 1];
@@ -399,7 +409,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
             const int m = mb + q * 8 + rd_row;
             if (R && (!GUARD || (m < p.M && n < p.N))) {
                 const float *rp = R + (int64_t)m * p.r_sm + n;
-                if (p.vec_r && n_in) res[q] = *reinterpret_cast<const f32x4 *>(rp);
+                if (!GUARD || (p.vec_r && n_in)) res[q] = *reinterpret_cast<const f32x4 *>(rp);
                 else {
                     res[q].x = rp[0];
                     if (n + 1 < p.N) res[q].y = rp[1];
@@ -428,27 +438,34 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         const int mb = m0 + wm * WM + (blk / TN) * 32, n = n0 + wn * WN + (blk % TN) * 32 + rd_col;
         const bool n_in = !GUARD || n + 3 < p.N;
+        // The row groups of the block: stage -> alpha, bias, activation, residual, activation -> C.  The launches
+        // without an activation (most of them) take a copy of the loop that has no activation code at all.
+        auto row_groups = [&](auto with_act) {
+            constexpr bool ACT = decltype(with_act)::value;
 #pragma unroll 1
-        for (int q = 0; q < 4; ++q) {
-            const int row = q * 8 + rd_row, m = mb + row;
-            f32x4 v = *reinterpret_cast<const f32x4 *>(&stage[row * STAGE_LD + rd_col]);
-            const f32x4 res = res_c[0];
-            res_c[0] = res_c[1]; res_c[1] = res_c[2]; res_c[2] = res_c[3];
-            if (GUARD && (m >= p.M || n >= p.N)) continue;
-            if (p.alpha != 1.0f) v *= p.alpha;
-            if (p.bias) v += bias_c;
-            if (p.act != SG_ACT_NONE) { v.x = apply_act(v.x, p.act); v.y = apply_act(v.y, p.act); v.z = apply_act(v.z, p.act); v.w = apply_act(v.w, p.act); }
-            if (R) v += res;
-            if (p.act_post != SG_ACT_NONE) { v.x = apply_act(v.x, p.act_post); v.y = apply_act(v.y, p.act_post); v.z = apply_act(v.z, p.act_post); v.w = apply_act(v.w, p.act_post); }
-            float *cp = C + (int64_t)m * p.c_sm + n;
-            if (p.vec_c && n_in) *reinterpret_cast<f32x4 *>(cp) = v;
-            else {
-                cp[0] = v.x;
-                if (n + 1 < p.N) cp[1] = v.y;
-                if (n + 2 < p.N) cp[2] = v.z;
-                if (n + 3 < p.N) cp[3] = v.w;
+            for (int q = 0; q < 4; ++q) {
+                const int row = q * 8 + rd_row, m = mb + row;
+                f32x4 v = *reinterpret_cast<const f32x4 *>(&stage[row * STAGE_LD + rd_col]);
+                const f32x4 res = res_c[0];
+                res_c[0] = res_c[1]; res_c[1] = res_c[2]; res_c[2] = res_c[3];
+                if (GUARD && (m >= p.M || n >= p.N)) continue;
+                if (p.alpha != 1.0f) v *= p.alpha;
+                if (p.bias) v += bias_c;
+                if (ACT) apply_act4(v, p.act);
+                if (R) v += res;
+                if (ACT) apply_act4(v, p.act_post);
+                float *cp = C + (int64_t)m * p.c_sm + n;
+                if (!GUARD || (p.vec_c && n_in)) *reinterpret_cast<f32x4 *>(cp) = v;
+                else {
+                    cp[0] = v.x;
+                    if (n + 1 < p.N) cp[1] = v.y;
+                    if (n + 2 < p.N) cp[2] = v.z;
+                    if (n + 3 < p.N) cp[3] = v.w;
+                }
             }
-        }
+        };
+        if (p.act == SG_ACT_NONE && p.act_post == SG_ACT_NONE) row_groups(std::false_type{});
+        else row_groups(std::true_type{});
         if (TM * TN > 1) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) res_c[q] = res_n[q];
@@ -519,7 +536,8 @@ bool needs_guard(const GemmP &p, int bm, int bn, bool a_kc, bool b_nc) {
     const int64_t span_a = a_kc ? (int64_t)bm * p.a_sm + BK : (int64_t)BK * p.a_sk + bm;
     const int64_t span_b = b_nc ? (int64_t)BK * p.b_sk + bn : (int64_t)bn * p.b_sn + BK;
     const bool fits32 = span_a >= 0 && span_b >= 0 && span_a < (1ll << 29) && span_b < (1ll << 29);
-    return p.M % bm != 0 || p.N % bn != 0 || p.K % (2 * BK) != 0 || !p.vec_a || !p.vec_b || !fits32;
+    const bool vec_out = p.vec_c && (!p.res || p.vec_r) && (!p.bias || p.vec_bias);
+    return p.M % bm != 0 || p.N % bn != 0 || p.K % (2 * BK) != 0 || !p.vec_a || !p.vec_b || !vec_out || !fits32;
 }
 
 // How many k ranges to split into.  Splitting pays when the output has too few tiles to occupy the
@@ -568,7 +586,7 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
             q.bias = nullptr; q.res = nullptr; q.alpha = 1.0f; q.act = SG_ACT_NONE; q.act_post = SG_ACT_NONE;
             q.vec_c = p.N % 4 == 0;
             dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, (unsigned)nsplit);
-            if (needs_guard(p, BM, BN, a_kc, b_nc)) launch_layouts<BM, BN, WAVES_M, true>(ctx, q, grid, a_kc, b_nc);
+            if (needs_guard(q, BM, BN, a_kc, b_nc)) launch_layouts<BM, BN, WAVES_M, true>(ctx, q, grid, a_kc, b_nc);
             else launch_layouts<BM, BN, WAVES_M, false>(ctx, q, grid, a_kc, b_nc);
             SG_CHECK_LAUNCH(ctx, "gemm (split-K pass 1)");
             const bool vec = p.N % 4 == 0;

@@ -38,6 +38,9 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));  // native vector: stays in registers
 
 constexpr int BK = 16;   // k-slab
+#ifndef SG_AGPR
+#define SG_AGPR 0
+#endif
 #ifndef SG_KPAD
 #define SG_KPAD 4
 #endif
@@ -109,24 +112,28 @@ template <int ROWS, bool K_CONTIG> struct Tile {
     }
     __device__ static __forceinline__ int lds_at(int row, int k) { return K_CONTIG ? row * LD + k : k * LD + row; }
 
-    // Unguarded loads (whole tile inside the matrix, 16-byte aligned) address an item as
-    //   uniform tile/slab base (scalar registers)  +  a per-lane 32-bit byte offset fixed for the kernel,
-    // so the K loop spends no vector instructions on addresses: lane_offset() is computed once per
-    // item before the loop, slab_base() is scalar arithmetic per slab.
+    // Unguarded loads (whole tile inside the matrix, 16-byte aligned) are buffer loads: the descriptor holds
+    // the tile's base address, the instruction takes a per-lane 32-bit byte offset that is fixed for the
+    // kernel (lane_offset(), computed once per item before the loop) and a scalar byte offset for the
+    // slab (slab_offset(), one scalar multiply per slab).  The K loop spends no vector instruction and
+    // no 64-bit arithmetic on addresses.
     __device__ static __forceinline__ uint32_t lane_offset(int i, uint32_t s_row, uint32_t s_k, int tid) {
         const int f = slot(tid + i * NTHREADS);
         int row, k;
         where(f, row, k);
         return (K_CONTIG ? (uint32_t)row * s_row + (uint32_t)k : (uint32_t)k * s_k + (uint32_t)row) * 4u;
     }
-    __device__ static __forceinline__ const char *tile_base(const float *base, int row0, int64_t s_row) {
-        return reinterpret_cast<const char *>(K_CONTIG ? base + (int64_t)row0 * s_row : base + row0);
+    __device__ static __forceinline__ const float *tile_base(const float *base, int row0, int64_t s_row) {
+        return K_CONTIG ? base + (int64_t)row0 * s_row : base + row0;
     }
-    __device__ static __forceinline__ const char *slab_base(const char *tile, int k0, int64_t s_k) {
-        return tile + (K_CONTIG ? (int64_t)k0 : (int64_t)k0 * s_k) * 4;
+    __device__ static __forceinline__ __amdgpu_buffer_rsrc_t descriptor(const float *tile) {
+        // raw buffer, stride 0, no range limit (the host checked that every offset stays below 2^31), 32-bit data format
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(tile), 0, -1, 0x00020000);
     }
-    __device__ static __forceinline__ void load_one_fast(f32x4 &r, const char *slab, uint32_t lane_off) {
-        r = *reinterpret_cast<const f32x4 *>(slab + lane_off);
+    __device__ static __forceinline__ uint32_t slab_offset(int k0, uint32_t s_k) { return (uint32_t)k0 * (K_CONTIG ? 4u : s_k * 4u); }
+    __device__ static __forceinline__ void load_one_fast(f32x4 &r, __amdgpu_buffer_rsrc_t tile, uint32_t lane_off, uint32_t slab_off) {
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+        r = __builtin_bit_cast(f32x4, (u32x4)__builtin_amdgcn_raw_buffer_load_b128(tile, lane_off, slab_off, 0));
     }
 
     // guarded: zero-fill outside [row_lim) x [k_lim), scalar loads when 16-byte loads are not legal
@@ -252,7 +259,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     for (int i = 0; i < TA::NV; ++i) off_a[i] = TA::lane_offset(i, (uint32_t)p.a_sm, (uint32_t)p.a_sk, tid);
 #pragma unroll
     for (int i = 0; i < TB::NV; ++i) off_b[i] = TB::lane_offset(i, (uint32_t)p.b_sn, (uint32_t)p.b_sk, tid);
-    const char *a_tile = TA::tile_base(A, m0, p.a_sm), *b_tile = TB::tile_base(B, n0, p.b_sn);
+    const __amdgpu_buffer_rsrc_t a_tile = TA::descriptor(TA::tile_base(A, m0, p.a_sm)), b_tile = TB::descriptor(TB::tile_base(B, n0, p.b_sn));
 
     // item e of a slab: global memory -> registers
 #define SG_ITEM_LOAD(e, RA, RB, k0)                                                            \
@@ -260,11 +267,11 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
         if ((e) < TA::NV) {                                                                    \
             const int ia = (e) < TA::NV ? (e) : 0;                                         \
             if (GUARD) TA::load_one_guarded(RA[ia], ia, A, m0, (k0), p.M, Kloc, p.a_sm, p.a_sk, p.vec_a, tid); \
-            else TA::load_one_fast(RA[ia], TA::slab_base(a_tile, (k0), p.a_sk), off_a[ia]);    \
+            else TA::load_one_fast(RA[ia], a_tile, off_a[ia], TA::slab_offset((k0), (uint32_t)p.a_sk)); \
         } else {                                                                               \
             const int ib = (e) >= TA::NV ? (e) - TA::NV : 0;                               \
             if (GUARD) TB::load_one_guarded(RB[ib], ib, B, n0, (k0), p.N, Kloc, p.b_sn, p.b_sk, p.vec_b, tid); \
-            else TB::load_one_fast(RB[ib], TB::slab_base(b_tile, (k0), p.b_sk), off_b[ib]);    \
+            else TB::load_one_fast(RB[ib], b_tile, off_b[ib], TB::slab_offset((k0), (uint32_t)p.b_sk)); \
         }                                                                                      \
     } while (0)
     // item e of a slab: registers -> LDS buffer BUF
@@ -289,10 +296,15 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
             TB::fetch(lds_b[BUF], b_col + ib * 32, G, khalf, BR[ib]);                          \
         }                                                                                      \
     } while (0)
+#if SG_AGPR
+#define SG_MFMA_OP(ACC, A_, B_) asm volatile("v_mfma_f32_32x32x2_f32 %0, %1, %2, %0" : "+a"(ACC) : "v"(A_), "v"(B_))
+#else
+#define SG_MFMA_OP(ACC, A_, B_) ACC = __builtin_amdgcn_mfma_f32_32x32x2f32(A_, B_, ACC, 0, 0, 0)
+#endif
 #define SG_MFMA(t, AR, BR)                                                                     \
     do {                                                                                       \
         const int s_ = (t) / (TM * TN), i_ = ((t) / TN) % TM, j_ = (t) % TN;               \
-        acc[i_][j_] = __builtin_amdgcn_mfma_f32_32x32x2f32(AR[i_][s_], BR[j_][s_], acc[i_][j_], 0, 0, 0); \
+        SG_MFMA_OP(acc[i_][j_], AR[i_][s_], BR[j_][s_]);                                      \
     } while (0)
 
     // Software pipeline of one wavefront, per K slab of 16 (two groups g0, g1 of four MFMA k-steps):
@@ -318,10 +330,15 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     // LDS queue draining.  (Measured against the other groupings and orders on the BERT and 4096^3
     // shapes: coarser groups starve the matrix pipe while a wavefront issues memory instructions, finer
     // ones for reads and requests were slower too.)
-    constexpr int W_PER = 1, R_PER = 2, G_PER = 2;
+#ifndef SG_WPER
+#define SG_WPER 1
+#define SG_RPER 2
+#define SG_GPER 2
+#endif
+    constexpr int W_PER = SG_WPER, R_PER = SG_RPER, G_PER = SG_GPER;
     constexpr int SW = (NWR + W_PER - 1) / W_PER, SR = (NRB + R_PER - 1) / R_PER;
-    static_assert(SW + SR + (NWR + G_PER - 1) / G_PER <= NMFMA, "more memory items than MFMA slots in a group");
-    auto slot3 = [](int e) constexpr { return e < NWR ? e / W_PER : e < NWR + NRB ? SW + (e - NWR) / R_PER : SW + SR + (e - NWR - NRB) / G_PER; };
+    // (items that find no slot of their own go behind the last MFMA of the group)
+    auto slot3 = [](int e) constexpr { const int t = e < NWR ? e / W_PER : e < NWR + NRB ? SW + (e - NWR) / R_PER : SW + SR + (e - NWR - NRB) / G_PER; return t < NMFMA ? t : NMFMA - 1; };
     constexpr int IPS5 = (NRB + NMFMA - 2) / (NMFMA - 1);
     // The body is unconditional: past the end of K the write goes to a buffer nobody reads again
     // and the fetch re-reads the last slab (unguarded path) or returns zeros (guarded path).  The
@@ -370,6 +387,9 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
         SG_SLAB_BODY(kt, ra1, rb1);
         SG_SLAB_BODY(kt + 1, ra0, rb0);
     }
+#if SG_AGPR
+    asm volatile("s_nop 15\n\ts_nop 15");  // the last MFMA's result is not interlocked against the reads below
+#endif
 #undef SG_SLAB_BODY
 #undef SG_ITEM_LOAD
 #undef SG_ITEM_STORE
@@ -532,10 +552,11 @@ void launch_layouts(sg_ctx *ctx, const GemmP &p, dim3 grid, bool a_kc, bool b_nc
 
 // GUARD = false needs every tile to lie fully inside the matrices and 16-byte loads to be legal.
 bool needs_guard(const GemmP &p, int bm, int bn, bool a_kc, bool b_nc) {
-    // the unguarded loads keep per-lane offsets inside a tile slab in 32 bits
-    const int64_t span_a = a_kc ? (int64_t)bm * p.a_sm + BK : (int64_t)BK * p.a_sk + bm;
-    const int64_t span_b = b_nc ? (int64_t)BK * p.b_sk + bn : (int64_t)bn * p.b_sn + BK;
-    const bool fits32 = span_a >= 0 && span_b >= 0 && span_a < (1ll << 29) && span_b < (1ll << 29);
+    // the unguarded loads address a tile through 32-bit byte offsets (per lane inside a slab, scalar per
+    // slab): everything a tile reaches over the whole of K must stay below 2^31 bytes from its base
+    const int64_t reach_a = a_kc ? (int64_t)bm * p.a_sm + p.K : (int64_t)p.K * p.a_sk + bm;
+    const int64_t reach_b = b_nc ? (int64_t)p.K * p.b_sk + bn : (int64_t)bn * p.b_sn + p.K;
+    const bool fits32 = reach_a >= 0 && reach_b >= 0 && reach_a < (1ll << 29) && reach_b < (1ll << 29);
     const bool vec_out = p.vec_c && (!p.res || p.vec_r) && (!p.bias || p.vec_bias);
     return p.M % bm != 0 || p.N % bn != 0 || p.K % (2 * BK) != 0 || !p.vec_a || !p.vec_b || !vec_out || !fits32;
 }

@@ -69,9 +69,28 @@ struct GemmP {
     int64_t c_sz;     // split-K: element stride between the partial results of consecutive z
 };
 
+// erf by the five-term rational-exponential form (Abramowitz & Stegun 7.1.26):
+//   erf(x) = 1 - (a1 t + .. + a5 t^5) exp(-x^2),  t = 1 / (1 + p x),  x >= 0,  odd in x,
+// with the hardware reciprocal and 2^x.  Absolute error below 6e-7 in fp32 (1.5e-7 from the formula, the
+// rest from forming 1 - small in fp32): three orders of magnitude inside the tolerance of a GEMM-bearing
+// result.  A dozen instructions, no branch, against about forty with two divergent paths for the
+// library routine; in an epilogue every vector instruction is a cycle taken from the matrix pipe.
+// The map kernels keep the exact routine.
+__device__ __forceinline__ float erf_short(float x) {
+    const float ax = __builtin_fabsf(x);
+    const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f, ax, 1.0f));
+    float q = __builtin_fmaf(1.061405429f, t, -1.453152027f);
+    q = __builtin_fmaf(q, t, 1.421413741f);
+    q = __builtin_fmaf(q, t, -0.284496736f);
+    q = __builtin_fmaf(q, t, 0.254829592f);
+    q *= t;
+    const float e = __builtin_amdgcn_exp2f(ax * ax * -1.44269504088896340736f);
+    return __builtin_copysignf(__builtin_fmaf(-q, e, 1.0f), x);
+}
+
 __device__ __forceinline__ float apply_act(float v, int act) {
     if (act == SG_ACT_RELU) return v > 0.0f ? v : 0.0f * v;  // (float)(v>0) * v, nn.rs:39
-    if (act == SG_ACT_GELU_ERF) return (v * 0.5f) * (erff(v * 0.70710678118654752440f) + 1.0f);
+    if (act == SG_ACT_GELU_ERF) return (v * 0.5f) * (erf_short(v * 0.70710678118654752440f) + 1.0f);
     return v;
 }
 // the same for the four values of a lane, with one uniform branch on the kind instead of four

@@ -45,9 +45,6 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));  // native vector: stays in registers
 
 constexpr int BK = 16;   // k-slab
-#ifndef SG_AGPR
-#define SG_AGPR 0
-#endif
 #ifndef SG_KPAD
 #define SG_KPAD 4
 #endif
@@ -332,11 +329,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
             TB::fetch(lds_b[BUF], b_col + ib * 32, G, khalf, BR[ib]);                          \
         }                                                                                      \
     } while (0)
-#if SG_AGPR
-#define SG_MFMA_OP(ACC, A_, B_) asm volatile("v_mfma_f32_32x32x2_f32 %0, %1, %2, %0" : "+a"(ACC) : "v"(A_), "v"(B_))
-#else
 #define SG_MFMA_OP(ACC, A_, B_) ACC = __builtin_amdgcn_mfma_f32_32x32x2f32(A_, B_, ACC, 0, 0, 0)
-#endif
 #define SG_MFMA(t, AR, BR)                                                                     \
     do {                                                                                       \
         const int s_ = (t) / (TM * TN), i_ = ((t) / TN) % TM, j_ = (t) % TN;               \
@@ -363,15 +356,9 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     constexpr int ITEMS3 = 2 * NWR + NRB;
     // Which MFMA of S3 an item is issued behind: LDS writes one per MFMA from the first, then LDS reads
     // two per MFMA, then global requests two per MFMA; the remaining MFMAs of the group run with the
-    // LDS queue draining.  (Measured against the other groupings and orders on the BERT and 4096^3
-    // shapes: coarser groups starve the matrix pipe while a wavefront issues memory instructions, finer
-    // ones for reads and requests were slower too.)
-#ifndef SG_WPER
-#define SG_WPER 1
-#define SG_RPER 2
-#define SG_GPER 2
-#endif
-    constexpr int W_PER = SG_WPER, R_PER = SG_RPER, G_PER = SG_GPER;
+    // LDS queue draining.  (Measured in cycles per slab of a 128x96 tile against other groupings: two
+    // LDS writes per MFMA +118, one global request per MFMA +24, all four requests behind one MFMA -10.)
+    constexpr int W_PER = 1, R_PER = 2, G_PER = 2;
     constexpr int SW = (NWR + W_PER - 1) / W_PER, SR = (NRB + R_PER - 1) / R_PER;
     // (items that find no slot of their own go behind the last MFMA of the group)
     auto slot3 = [](int e) constexpr { const int t = e < NWR ? e / W_PER : e < NWR + NRB ? SW + (e - NWR) / R_PER : SW + SR + (e - NWR - NRB) / G_PER; return t < NMFMA ? t : NMFMA - 1; };
@@ -423,14 +410,12 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
         SG_SLAB_BODY(kt, ra1, rb1);
         SG_SLAB_BODY(kt + 1, ra0, rb0);
     }
-#if SG_AGPR
-    asm volatile("s_nop 15\n\ts_nop 15");  // the last MFMA's result is not interlocked against the reads below
-#endif
 #undef SG_SLAB_BODY
 #undef SG_ITEM_LOAD
 #undef SG_ITEM_STORE
 #undef SG_ITEM_FETCH
 #undef SG_MFMA
+#undef SG_MFMA_OP
 
     // ---- epilogue.  Element r of a 32x32 accumulator block sits at row (r/4)*8 + (lane/32)*4 + r%4,
     // column lane%32.  Each wavefront passes its blocks one at a time through a private 32x32 LDS

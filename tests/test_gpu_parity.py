@@ -367,6 +367,24 @@ def test_gemm_split_k(ctx, monkeypatch, mkn, split, ta, tb):
     exact(y2, y3, "run-to-run")
 
 
+@pytest.mark.parametrize("mkn", [(3200, 64, 3840), (3201, 96, 3838), (4096, 32, 2304)])
+def test_gemm_more_tiles_than_resident_workgroups(ctx, mkn):
+    """Outputs of 750..1000 tiles: more than the three workgroups per compute unit that fit at once, so
+    workgroups take a second tile (exactly tiled shapes through buffer loads, the ragged one through the
+    guarded loads).  Every element against float64, and the same bits on a second run."""
+    m, k, n = mkn
+    say("gemm tile walk", mkn)
+    rng = np.random.default_rng(m + n)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (n,)).astype(np.float32)
+    res = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    run = lambda: ((dev(ctx, a).matmul(dev(ctx, b)) + dev(ctx, bias)) + dev(ctx, res)).eval(ctx).numpy()
+    y = run()
+    close(y, a.astype(np.float64) @ b.astype(np.float64) + bias + res, REL_GEMM, "vs float64")
+    exact(y, run(), "run-to-run")
+
+
 def test_gemm_batched_split_k(ctx, monkeypatch):
     say("gemm_batched split-K")
     monkeypatch.setenv("SAGE_GEMM_SPLITK", "4")

@@ -201,6 +201,8 @@ RED_CASES = [
     ((2, 3, 2, 3, 2), [0, 2, 3]), ((6, 7, 8), [0, 1, 2]), ((4, 6, 10), [2, 0]), ((128, 128), [1]), ((1, 7), [0]),
     # few contiguous outputs, long strided reduced axis (bias gradients): chunked column path
     ((5000, 70), [0]), ((6272, 64), [0]), ((3, 400, 513), [0, 1]), ((300, 16), [0]),
+    # row lengths that leave some lanes out of the four-loads-per-trip loop and in its one-load tail
+    ((7, 1000), [1]), ((4, 1900), [1]), ((3, 2052), [1]),
 ]
 
 

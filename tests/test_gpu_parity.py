@@ -387,6 +387,41 @@ def test_gemm_more_tiles_than_resident_workgroups(ctx, mkn):
     exact(y, run(), "run-to-run")
 
 
+def test_gemm_random_shapes_and_layouts(ctx):
+    """Sixty seeded random products: extents 1..400 (most of them ragged against every tile size), all four
+    transpose modes, operands that are row windows of larger matrices (element offsets, ld > width), with
+    and without bias / ReLU / residual.  Against float64 and against the oracle."""
+    rng = np.random.default_rng(2024)
+    for case in range(60):
+        m, n, k = (int(rng.integers(1, 401)) for _ in range(3))
+        if case % 7 == 0:
+            m, n, k = 128 * int(rng.integers(1, 4)), 96 * int(rng.integers(1, 4)), 32 * int(rng.integers(1, 9))  # exactly tiled
+        ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        pad_a, pad_b = int(rng.integers(0, 3)), int(rng.integers(0, 3))
+        sa = (k, m) if ta else (m, k)
+        sb = (n, k) if tb else (k, n)
+        big_a = rng.uniform(-1, 1, (sa[0] + 2 * pad_a, sa[1])).astype(np.float32)
+        big_b = rng.uniform(-1, 1, (sb[0] + 2 * pad_b, sb[1])).astype(np.float32)
+        say("gemm random", case, (m, n, k), ta, tb, pad_a, pad_b)
+        ad, ao = view_pair(ctx, big_a, lambda t: t.slice(0, pad_a, pad_a + sa[0]))
+        bd, bo = view_pair(ctx, big_b, lambda t: t.slice(0, pad_b, pad_b + sb[0]))
+        a64 = big_a[pad_a:pad_a + sa[0]].astype(np.float64)
+        b64 = big_b[pad_b:pad_b + sb[0]].astype(np.float64)
+        ref = (a64.T if ta else a64) @ (b64.T if tb else b64)
+        y = V.gemm(ad, bd, ta, tb)
+        yo = O.gemm(ao, bo, ta, tb)
+        kind = case % 3
+        if kind >= 1:
+            bias = rng.uniform(-1, 1, (n,)).astype(np.float32)
+            y, yo, ref = y + dev(ctx, bias), O.binary("add", yo, ht(bias).expand([m, n])), ref + bias
+        if kind == 2:
+            res = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+            y, yo, ref = nn.relu(y) + dev(ctx, res), O.binary("add", O.relu(yo), ht(res)), np.maximum(ref, 0) + res
+        out = y.eval(ctx).numpy()
+        close(out, ref, REL_GEMM, f"case {case} vs float64")
+        close(out, yo.numpy(), REL_GEMM, f"case {case} vs oracle")
+
+
 def test_gemm_batched_split_k(ctx, monkeypatch):
     say("gemm_batched split-K")
     monkeypatch.setenv("SAGE_GEMM_SPLITK", "4")

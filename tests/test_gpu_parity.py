@@ -743,6 +743,35 @@ def test_layer_norm(ctx, shape, per_feature):
     close(yf, yo, 5e-4, "fused vs oracle")
 
 
+ROW_LENGTHS = [1, 3, 4, 7, 16, 17, 32, 36, 64, 68, 100, 128, 132, 200, 256, 260, 384, 512, 516, 768, 1000, 1024, 1028, 1536, 2048, 2052, 2100]
+
+
+@pytest.mark.parametrize("length", ROW_LENGTHS)
+def test_row_kernels_every_dispatch_class(ctx, length):
+    """softmax (with a per-row addend), softmax cross-entropy and LayerNorm at row lengths on both sides of
+    every lanes-per-row / chunks-per-lane boundary of the row kernels, plus lengths no vector path takes;
+    37 rows, so the last wavefront is partly empty."""
+    say("row kernels", length)
+    rng = np.random.default_rng(length)
+    rows = 37
+    x = (rng.standard_normal((rows, length)) * 2).astype(np.float32)
+    add = rng.standard_normal((rows, 1)).astype(np.float32)
+    close(nn.softmax(dev(ctx, x) + dev(ctx, add), 1).eval(ctx).numpy(), O.softmax(O.binary("add", ht(x), ht(add).expand([rows, length])), 1).numpy(),
+          REL_MAP, "softmax")
+    lab = rng.integers(0, length, (rows, 1)).astype(np.int32)
+    loss = nn.softmax_cross_entropy(dev(ctx, x), dev(ctx, lab)).eval(ctx).numpy()
+    loss_o = O.softmax_cross_entropy(ht(x), ht(lab.view(np.uint32))).numpy()
+    if length == 1:  # one class: the loss is 0 up to the rounding of log(exp(x)); nothing to scale a relative bound by
+        assert np.max(np.abs(loss - loss_o)) < 1e-6
+    else:
+        close(loss, loss_o, REL_MAP, "softmax_cross_entropy")
+    if length > 1:
+        g = rng.uniform(0.5, 1.5, (length,)).astype(np.float32)
+        b = rng.standard_normal((length,)).astype(np.float32)
+        close(nn.layer_norm(dev(ctx, x), 1, dev(ctx, g), dev(ctx, b), 1e-5).eval(ctx).numpy(), O.layer_norm(ht(x), 1, ht(g), ht(b), 1e-5).numpy(),
+              5e-4, "layer_norm")
+
+
 # ----------------------------------------------------------------------------- random fills
 @pytest.mark.parametrize("shape", [(3, 3), (1000,), (7, 11, 13), (1 << 20,)])
 def test_rand_uniform_and_normal(ctx, shape):

@@ -137,3 +137,29 @@ def test_config5_bert_layer_b64_s512_batch_slice(ctx):
     z = (y_full.astype(np.float64) - p["ln2_b"]) / p["ln2_g"]
     assert np.abs(z.mean(-1)).max() < 1e-3
     close(z.var(-1), np.ones(z.shape[:2]), REL_GEMM, "rows normalised")
+
+
+def test_streamed_maps_at_full_size_are_exact(ctx):
+    """Maps whose operands total more than the streaming threshold take non-temporal loads and stores:
+    the three-input (g + bias) + x map of a BERT layer at [4096, 3072] (151 MB) and a strided-operand
+    map of the same size are bit-exact against numpy, the exp(x - c) map of config 1 (67 MB) matches the
+    oracle; the same expressions on a small tensor (regular accesses) agree with their full-size rows."""
+    rng = np.random.default_rng(12)
+    m, n = 4096, 3072
+    g = rng.standard_normal((m, n)).astype(np.float32)
+    x = rng.standard_normal((m, n)).astype(np.float32)
+    bias = rng.standard_normal((n,)).astype(np.float32)
+    say("streamed (g+bias)+x", (m, n))
+    y = ((dev(ctx, g) + dev(ctx, bias)) + dev(ctx, x)).eval(ctx).numpy()
+    assert np.array_equal(y, (g + bias) + x)
+    small = ((dev(ctx, g[:8]) + dev(ctx, bias)) + dev(ctx, x[:8])).eval(ctx).numpy()
+    assert np.array_equal(small, y[:8])
+    say("streamed map with a transposed operand", (n, m))
+    yt = (dev(ctx, g).transpose(0, 1) * 2.0 + dev(ctx, x.T.copy())).eval(ctx).numpy()
+    assert np.array_equal(yt, g.T * np.float32(2.0) + x.T)
+    say("streamed exp(x - c)", (8192, 1024))
+    lg = rng.standard_normal((8192, 1024)).astype(np.float32)
+    c = lg.max(1, keepdims=True)
+    e = (dev(ctx, lg) - dev(ctx, c)).exp().eval(ctx).numpy()
+    close(e[:64], O.unary("exp", O.binary("sub", ht(lg[:64]), ht(c[:64]).expand([64, 1024]))).numpy(), REL_MAP, "rows vs oracle")
+    assert np.all(e <= 1.0) and np.all(e.max(1) == 1.0)

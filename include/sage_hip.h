@@ -208,7 +208,7 @@ typedef struct sg_gemm_epilogue {
     int32_t act;               /* sg_act, applied after bias */
     int32_t act_post;          /* sg_act, applied after residual */
     const sg_tensor *bias;     /* numel == N, unit stride, or NULL */
-    const sg_tensor *residual; /* same extents as C, last stride 1, or NULL */
+    const sg_tensor *residual; /* [M,N], [batch,M,N] (batch axes flattened) or C's extents; last stride 1; or NULL */
 } sg_gemm_epilogue;
 
 /* (A long-K product with few output tiles uses a workspace from the context allocator: SG_ERR_OOM when it does not fit.)

@@ -45,14 +45,8 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));  // native vector: stays in registers
 
 constexpr int BK = 16;   // k-slab
-#ifndef SG_KPAD
-#define SG_KPAD 4
-#endif
-#ifndef SG_RPAD
-#define SG_RPAD 4
-#endif
-constexpr int KPAD = SG_KPAD;  // row padding of [row][k] LDS tiles (floats)
-constexpr int RPAD = SG_RPAD;  // row padding of [k][row] LDS tiles (floats)
+constexpr int KPAD = 4;  // row padding of [row][k] LDS tiles (floats)
+constexpr int RPAD = 4;  // row padding of [k][row] LDS tiles (floats)
 constexpr int NTHREADS = 256;
 constexpr int NUM_XCD = 8;
 
@@ -741,7 +735,7 @@ int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c,
             int rc = sg_validate_tensor(ctx, t, "gemm residual");
             if (rc != SG_OK) return rc;
             if (t->dtype != SG_FLOAT) return sg_fail(ctx, SG_ERR_DTYPE, "gemm: residual must be fp32");
-            // accepted layouts: [M,N] for a single matrix, or the same rank as C
+            // accepted layouts: [M,N] for a single matrix, [batch,M,N] with the batch axes flattened, or [b0,b1,M,N]
             const int r = t->rank;
             if (r < 2 || t->extents[r - 1] != N || t->extents[r - 2] != M || (N != 1 && t->strides[r - 1] != 1))
                 return sg_fail(ctx, SG_ERR_SHAPE, "gemm: residual must be [..,M,N] with unit last stride");
@@ -752,9 +746,9 @@ int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c,
             p.r_sm = t->strides[r - 2];
             p.r_sb1 = r >= 3 ? t->strides[r - 3] : 0;
             p.r_sb0 = r >= 4 ? t->strides[r - 4] : 0;
-            if (r == 3 && nb0 > 1) {  // a single batch axis on the residual while C has it in b0
-                p.r_sb0 = t->strides[0];
-                p.r_sb1 = 0;
+            if (r == 3) {  // one flattened batch axis: entry b0 * nb1 + b1
+                p.r_sb1 = t->strides[0];
+                p.r_sb0 = (int64_t)nb1 * t->strides[0];
             }
             if (r > 4) return sg_fail(ctx, SG_ERR_SHAPE, "gemm: residual rank above 4");
             p.vec_r = (N == 1 || t->strides[r - 1] == 1) && ptr_aligned16(p.res) && mult4(p.r_sm) && mult4(p.r_sb0) && mult4(p.r_sb1);

@@ -76,6 +76,7 @@ int sg_ctx_create(int device_idx, uint64_t capacity_bytes, sg_ctx **out) {
 int sg_trim(sg_ctx *ctx) {
     if (!ctx) return SG_ERR_ARG;
     if (ctx->cache.empty()) return SG_OK;
+    if (ctx->capturing) return sg_fail(ctx, SG_ERR_ARG, "sg_trim waits for the stream and cannot be captured into a graph");
     SG_HIP(ctx, hipStreamSynchronize(ctx->stream));
     for (auto &kv : ctx->cache) {
         (void)hipFree(kv.second);

@@ -217,6 +217,20 @@ typedef struct sg_gemm_epilogue {
  * be 1 (the reference organizes its inputs first, gemm.rs:111-112).  fp32 only. */
 int sg_gemm(sg_ctx *ctx, int transpose_a, int transpose_b, const sg_tensor *a, const sg_tensor *b,
             const sg_tensor *c, const sg_gemm_epilogue *epi);
+/* No counterpart in the reference.  For callers that cannot allocate device memory at the call:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same
+ * arguments, same kernels and bit-identical results as sg_gemm, but the split-K workspace of a
+ * few-tile/long-K product is a static array of SG_GEMM_NOALLOC_SCRATCH_BYTES in the library's code
+ * object (one copy per GPU, held until the process ends) instead of a block from the context's
+ * allocator; the call performs no allocation or free of any kind.  A product whose split-K partial
+ * products (ranges x M x N x 4 bytes) exceed the array returns SG_ERR_ARG and computes nothing.
+ * All contexts on one GPU share that GPU's array: calls that may overlap on one GPU (different
+ * contexts/streams, or two replays of graphs holding this call) race and must be serialised by
+ * the caller.  Nothing in the array needs clearing between calls: pass 1 overwrites every element
+ * pass 2 reads. */
+#define SG_GEMM_NOALLOC_SCRATCH_BYTES (32u << 20)
+int sg_gemm_noalloc(sg_ctx *ctx, int transpose_a, int transpose_b, const sg_tensor *a,
+                    const sg_tensor *b, const sg_tensor *c, const sg_gemm_epilogue *epi);
 /* GemmBatched::compute_direct (gemm.rs:338-421): rank 3, batch stride = strides[0], ld = strides[1]. */
 int sg_gemm_batched(sg_ctx *ctx, int transpose_a, int transpose_b, const sg_tensor *a,
                     const sg_tensor *b, const sg_tensor *c, const sg_gemm_epilogue *epi);

@@ -14,6 +14,7 @@ MAX_RANK = 8
 MAX_MAP_INPUTS = 16
 MAX_EXPR = 128
 REFERENCE_CAPACITY_BYTES = 1000 * 1024 * 1024
+GEMM_NOALLOC_SCRATCH_BYTES = 32 << 20
 
 OK, ERR_OOM, ERR_DEVICE, ERR_SHAPE, ERR_DTYPE, ERR_ARG = range(6)
 CHAR, SHORT, INT, LONG, UCHAR, USHORT, UINT, ULONG, FLOAT, HALF = range(10)
@@ -81,6 +82,7 @@ PROTOTYPES = {
     "sg_unslice": (C.c_int, [_CTX, C.c_int, C.c_int64, _TP, _TP]),
     "sg_concat": (C.c_int, [_CTX, C.c_int, _TP, C.c_int, _TP]),
     "sg_gemm": (C.c_int, [_CTX, C.c_int, C.c_int, _TP, _TP, _TP, C.POINTER(sg_gemm_epilogue)]),
+    "sg_gemm_noalloc": (C.c_int, [_CTX, C.c_int, C.c_int, _TP, _TP, _TP, C.POINTER(sg_gemm_epilogue)]),
     "sg_gemm_batched": (C.c_int, [_CTX, C.c_int, C.c_int, _TP, _TP, _TP, C.POINTER(sg_gemm_epilogue)]),
     "sg_matmul_strided": (C.c_int, [_CTX, _TP, _TP, _TP, C.POINTER(sg_gemm_epilogue)]),
     "sg_gemm_kernel_name": (C.c_int, [_CTX, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_char_p, C.c_uint64]),

@@ -99,6 +99,9 @@ static inline bool sg_is_dense(const sg_tensor *t) {
 
 int sg_validate_tensor(sg_ctx *ctx, const sg_tensor *t, const char *name);
 
+// gemm.hip: per-device set-up (the address of the static split-K scratch), run by sg_ctx_create.
+int sg_gemm_device_setup(sg_ctx *ctx);
+
 // A kernel that moves this many bytes streams them: past this size nothing it reads or writes is
 // found in the caches by its neighbours in the queue anyway, and non-temporal loads and stores
 // (no allocation in the L2s on the way through) sustain about a fifth more HBM bandwidth.

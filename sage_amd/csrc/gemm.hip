@@ -50,6 +50,14 @@ constexpr int RPAD = 4;  // row padding of [k][row] LDS tiles (floats)
 constexpr int NTHREADS = 256;
 constexpr int NUM_XCD = 8;
 
+// Split-K workspace of sg_gemm_noalloc: partial products [split][batch][M][N].  One copy per GPU,
+// held until the process ends.  In host code the name `scratch` is only a handle for
+// hipGetSymbolAddress; the address kernels and copies use is the per-device pointer below.
+constexpr int64_t SCRATCH_FLOATS = (int64_t)SG_GEMM_NOALLOC_SCRATCH_BYTES / 4;
+static __device__ __align__(256) float scratch[SCRATCH_FLOATS];
+constexpr int MAX_DEVICES = 64;
+float *g_scratch_ptr[MAX_DEVICES] = {};  // device address of `scratch` on each GPU, set by sg_gemm_device_setup
+
 struct GemmP {
     const float *A, *B;
     float *C;
@@ -602,7 +610,7 @@ int choose_split(int num_cus, int64_t wgs, int K, int *k_chunk) {
 }
 
 template <int BM, int BN, int WAVES_M>
-int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
+int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noalloc) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     int k_chunk = 0;
@@ -614,8 +622,17 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
         // eviction loop, session.rs:259-325, frees memory and calls again) instead of silently taking
         // the single-pass kernel, whose rounding differs: the same call always gives the same bits.
         void *ws = nullptr;
-        const int rc_ws = sg_alloc(ctx, (uint64_t)nsplit * slice * sizeof(float), &ws);
-        if (rc_ws != SG_OK) return rc_ws;
+        if (noalloc) {
+            // the per-device static array instead: nothing is allocated, larger products are refused
+            if ((int64_t)nsplit * slice > SCRATCH_FLOATS)
+                return sg_fail(ctx, SG_ERR_ARG, "sg_gemm_noalloc: this product runs split-K over %d ranges and needs %lld bytes of workspace, "
+                               "more than the %lld-byte static scratch (use sg_gemm)", nsplit, (long long)nsplit * slice * 4, (long long)SCRATCH_FLOATS * 4);
+            ws = ctx->device >= 0 && ctx->device < MAX_DEVICES ? g_scratch_ptr[ctx->device] : nullptr;
+            if (!ws) return sg_fail(ctx, SG_ERR_DEVICE, "sg_gemm_noalloc: the static scratch of device %d was not set up", ctx->device);
+        } else {
+            const int rc_ws = sg_alloc(ctx, (uint64_t)nsplit * slice * sizeof(float), &ws);
+            if (rc_ws != SG_OK) return rc_ws;
+        }
         {
             GemmP q = p;  // first pass: raw partial products into the workspace
             q.C = (float *)ws;
@@ -633,6 +650,7 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
             if (vec) hipLaunchKernelGGL((splitk_reduce_kernel<true>), rgrid, dim3(256), 0, ctx->stream, (const float *)ws, nsplit, slice, p, total);
             else hipLaunchKernelGGL((splitk_reduce_kernel<false>), rgrid, dim3(256), 0, ctx->stream, (const float *)ws, nsplit, slice, p, total);
             SG_CHECK_LAUNCH(ctx, "gemm (split-K pass 2)");
+            if (noalloc) return SG_OK;  // the static scratch stays; the next call on this stream is ordered behind pass 2
             // the block returns to the context's cache; later users are ordered behind these kernels on the stream
             return sg_free(ctx, ws);
         }
@@ -674,12 +692,12 @@ int choose_tile(int num_cus, int M, int N, int batch) {
     return best;
 }
 
-int launch_gemm(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc) {
+int launch_gemm(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noalloc) {
     switch (choose_tile(ctx->num_cus, p.M, p.N, batch)) {
-    case 0: return launch_cfg<128, 128, 2>(ctx, p, batch, a_kc, b_nc);
-    case 1: return launch_cfg<128, 96, 4>(ctx, p, batch, a_kc, b_nc);
-    case 2: return launch_cfg<128, 64, 2>(ctx, p, batch, a_kc, b_nc);
-    default: return launch_cfg<64, 64, 2>(ctx, p, batch, a_kc, b_nc);
+    case 0: return launch_cfg<128, 128, 2>(ctx, p, batch, a_kc, b_nc, noalloc);
+    case 1: return launch_cfg<128, 96, 4>(ctx, p, batch, a_kc, b_nc, noalloc);
+    case 2: return launch_cfg<128, 64, 2>(ctx, p, batch, a_kc, b_nc, noalloc);
+    default: return launch_cfg<64, 64, 2>(ctx, p, batch, a_kc, b_nc, noalloc);
     }
 }
 
@@ -691,7 +709,7 @@ struct Mat {
     int64_t sb0, sb1, s_row, s_col;
 };
 
-int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c, const sg_gemm_epilogue *epi) {
+int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c, const sg_gemm_epilogue *epi, bool noalloc = false) {
     if (M < 1 || N < 1 || K < 1) return sg_fail(ctx, SG_ERR_SHAPE, "gemm: empty dimension");
     // Which axis of each operand is the contiguous one.  An axis of extent 1 may carry any stride.
     bool a_kc, b_nc;
@@ -754,7 +772,7 @@ int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c,
             p.vec_r = (N == 1 || t->strides[r - 1] == 1) && ptr_aligned16(p.res) && mult4(p.r_sm) && mult4(p.r_sb0) && mult4(p.r_sb1);
         }
     }
-    return launch_gemm(ctx, p, nb0 * nb1, a_kc, b_nc);
+    return launch_gemm(ctx, p, nb0 * nb1, a_kc, b_nc, noalloc);
 }
 
 int check_f32(sg_ctx *ctx, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c, const char *who) {
@@ -779,8 +797,9 @@ extern "C" int sg_gemm_kernel_name(sg_ctx *ctx, int64_t M, int64_t N, int64_t K,
     return SG_OK;
 }
 
-extern "C" int sg_gemm(sg_ctx *ctx, int ta, int tb, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c,
-                       const sg_gemm_epilogue *epi) {
+namespace {
+int gemm_rank2(sg_ctx *ctx, int ta, int tb, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c, const sg_gemm_epilogue *epi,
+               bool noalloc) {
     if (!ctx) return SG_ERR_ARG;
     int rc = check_f32(ctx, a, b, c, "sg_gemm");
     if (rc != SG_OK) return rc;
@@ -796,7 +815,30 @@ extern "C" int sg_gemm(sg_ctx *ctx, int ta, int tb, const sg_tensor *a, const sg
     Mat ma{(const float *)a->base + a->offset, 0, 0, ta ? 1 : a->strides[0], ta ? a->strides[0] : 1};
     Mat mb{(const float *)b->base + b->offset, 0, 0, tb ? 1 : b->strides[0], tb ? b->strides[0] : 1};
     Mat mc{(const float *)c->base + c->offset, 0, 0, c->strides[0], 1};
-    return run(ctx, (int)M, (int)N, (int)K, 1, 1, ma, mb, mc, epi);
+    return run(ctx, (int)M, (int)N, (int)K, 1, 1, ma, mb, mc, epi, noalloc);
+}
+}  // namespace
+
+extern "C" int sg_gemm(sg_ctx *ctx, int ta, int tb, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c,
+                       const sg_gemm_epilogue *epi) {
+    return gemm_rank2(ctx, ta, tb, a, b, c, epi, false);
+}
+
+// The same product with the split-K workspace in the static per-device array: no allocation of any kind.
+extern "C" int sg_gemm_noalloc(sg_ctx *ctx, int ta, int tb, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c,
+                               const sg_gemm_epilogue *epi) {
+    return gemm_rank2(ctx, ta, tb, a, b, c, epi, true);
+}
+
+// Called by sg_ctx_create with the context's device current: resolves the device address of `scratch`
+// on that GPU once (each GPU holds its own copy of the array at its own address).
+int sg_gemm_device_setup(sg_ctx *ctx) {
+    if (ctx->device < 0 || ctx->device >= MAX_DEVICES) return SG_OK;  // sg_gemm_noalloc reports it when used
+    if (g_scratch_ptr[ctx->device]) return SG_OK;
+    float *ptr = nullptr;
+    SG_HIP(ctx, hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+    g_scratch_ptr[ctx->device] = ptr;
+    return SG_OK;
 }
 
 extern "C" int sg_gemm_batched(sg_ctx *ctx, int ta, int tb, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c,

@@ -69,6 +69,11 @@ int sg_ctx_create(int device_idx, uint64_t capacity_bytes, sg_ctx **out) {
         delete ctx;
         return SG_ERR_DEVICE;
     }
+    if (sg_gemm_device_setup(ctx) != SG_OK) {
+        (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return SG_ERR_DEVICE;
+    }
     *out = ctx;
     return SG_OK;
 }

@@ -45,13 +45,19 @@ def measured_traffic(kernel, workload):
         return None
 
 
-def build_bert(ctx, variant, batch, seq, layers, rng):
+def build_bert(ctx, variant, batch, seq, layers, rng, detail=False):
+    """The model the metric is quoted on.  variant "config": erf-GELU, LayerNorm eps 1e-12 with per-feature
+    gamma/beta, a 2-row segment table with segment ids, classifier on token 0.  variant "reference": what the
+    reference's models/bert.rs composes (ReLU, eps 1e-5, scalar gamma = beta = 1, no segment table, token 1).
+    detail=True also returns the host arrays (params() order), inputs and the last encoder output, for the
+    parity tests that rebuild the same model on the CPU."""
     import sage_amd as S
     from sage_amd.bert import Bert, BertConfig
     cfg = BertConfig.base()
     cfg.num_layers = layers
     exact = variant == "reference"
-    model = Bert(cfg, reference_exact=exact, segments=0)
+    model = Bert(cfg, reference_exact=exact, segments=0 if exact else 2)
+    arrays = []
     for p in model.params():
         n = p.label or ""
         if "layer_norm.gamma" in n:
@@ -62,12 +68,18 @@ def build_bert(ctx, variant, batch, seq, layers, rng):
             a = np.zeros(p.extents, np.float32)
         else:
             a = (rng.standard_normal(p.extents) * 0.02).astype(np.float32)
+        arrays.append(a)
         p.set(S.Tensor.from_numpy(ctx, a))
     ids = rng.integers(0, cfg.num_vocabs, (batch, seq)).astype(np.int32)
     mask = np.ones((batch, seq), np.float32)
+    seg = None if exact else rng.integers(0, 2, (batch, seq)).astype(np.int32)
     ids_v = S.Var.new(S.Tensor.from_numpy(ctx, ids))
     mask_v = S.Var.new(S.Tensor.from_numpy(ctx, mask))
-    logits = model.pass_(ids_v, mask_v, ctx)
+    seg_v = None if seg is None else S.Var.new(S.Tensor.from_numpy(ctx, seg))
+    hidden = model.encode(model.embedding.pass_(ids_v, ctx, seg_v), mask_v)
+    logits = model.classify(hidden)
+    if detail:
+        return {"cfg": cfg, "model": model, "logits": logits, "hidden": hidden, "arrays": arrays, "ids": ids, "mask": mask, "segment_ids": seg}
     return cfg, model, logits
 
 
@@ -489,7 +501,8 @@ def main():
     else:
         metric, unit = f"BERT-base fwd seqs/sec (b{a.batch},s{a.seq},fp32)", "seqs/s"
         config = {"workload": f"bert_base_forward_b{a.batch}_s{a.seq}_fp32", "variant": a.variant, "layers": a.layers,
-                  "hidden": cfg.embed_dim, "heads": cfg.num_attention_heads, "ffn": cfg.hidden_dim, "vocab": cfg.num_vocabs}
+                  "hidden": cfg.embed_dim, "heads": cfg.num_attention_heads, "ffn": cfg.hidden_dim, "vocab": cfg.num_vocabs,
+                  "segment_table_rows": 0 if a.variant == "reference" else 2}
     config.update({"replay": "hip_graph" if use_graph else "eager", "launches_per_step": len(prog.calls), "gemm_tflops_whole_step": total_gemm_flops / (ms_per_step * 1e-3) / 1e12})
     res = {
         "metric": metric,

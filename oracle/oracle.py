@@ -665,21 +665,29 @@ def bert_layer(x, mask, p, heads, act="relu", eps=1e-5):
     return layer_norm(binary("add", f, h1), [2], p["ln2_g"], p["ln2_b"], eps)
 
 
-def bert_embedding(ids, p, eps=1e-5):  # BertEmbedding::pass bert.rs:128-139
+def bert_embedding(ids, p, eps=1e-5, segment_ids=None):  # BertEmbedding::pass bert.rs:128-139
+    """word + position embeddings -> LayerNorm.  The reference has no segment table (bert.rs:97-102);
+    when p holds "seg_emb" and segment_ids is given, its rows are added the same way before the
+    LayerNorm (the benchmark's configuration variant)."""
     l = ids.extents[1]
     pos = HT.from_numpy(np.arange(l, dtype=np.uint32))
     we = embedding(p["word_emb"], ids)
     pe = embedding(p["pos_emb"], pos)
-    return layer_norm(binary("add", we, pe), [2], p["emb_g"], p["emb_b"], eps)
+    e = binary("add", we, pe)
+    if segment_ids is not None and "seg_emb" in p:
+        e = binary("add", e, embedding(p["seg_emb"], segment_ids))
+    return layer_norm(e, [2], p["emb_g"], p["emb_b"], eps)
 
 
-def bert_forward(ids, mask, p, heads, act="relu", eps=1e-5, cls_index=1):
-    """Bert::pass (bert.rs:72-81): classifier on token index 1."""
-    x = bert_embedding(ids, p, eps)
+def bert_forward(ids, mask, p, heads, act="relu", eps=1e-5, cls_index=1, segment_ids=None, return_hidden=False):
+    """Bert::pass (bert.rs:72-81): classifier on token index 1 (cls_index=0, act='gelu', eps=1e-12 and a
+    segment table give the benchmark's configuration variant from the same operators)."""
+    x = bert_embedding(ids, p, eps, segment_ids)
     for lp in p["layers"]:
         x = bert_layer(x, mask, lp, heads, act, eps)
     cls = x.index(1, cls_index).squeeze(1)
-    return dense(cls, p["wc"], p["bc"])
+    y = dense(cls, p["wc"], p["bc"])
+    return (y, x) if return_hidden else y
 
 
 # ----------------------------------------------------------------------------- ResNet (models/resnet.rs)

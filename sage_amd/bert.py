@@ -144,8 +144,11 @@ class Bert(Layer):
             x = l.pass_(x, attn_mask)
         return x
 
+    def classify(self, f):
+        """bert.rs:76-79: the classifier reads one token of the last encoder output."""
+        cls = f.index(1, 1 if self.reference_exact else 0).squeeze(1)
+        return self.classifier.pass_(cls)
+
     def pass_(self, token_ids, attn_mask, ctx, segment_ids=None):
         e = self.embedding.pass_(token_ids, ctx, segment_ids)
-        f = self.encode(e, into_var(attn_mask))
-        cls = f.index(1, 1 if self.reference_exact else 0).squeeze(1)  # bert.rs:76
-        return self.classifier.pass_(cls)
+        return self.classify(self.encode(e, into_var(attn_mask)))

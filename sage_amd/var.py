@@ -637,6 +637,11 @@ class _MapBuilder:
         self.prog.append((abi.EXPR_INPUT, self.keys[key], 0, 0))
 
 
+def fresh_seed():
+    """Two 32-bit seeds from the host's entropy, as the reference draws them per call (rand.rs:70, 113)."""
+    return tuple(int(b) for b in np.frombuffer(os.urandom(8), np.uint32))
+
+
 def refresh_derived(ctx, entries):
     """Re-run the calls that build cached derived data when parameters changed since they last ran."""
     for e in entries:
@@ -677,6 +682,7 @@ class Program:
         self._ev = _Evaluator(ctx, targets, record=self.calls)
         self.outputs = [self._ev.get(t) for t in targets]
         self.derived = self._ev.derived
+        self.reseed = self._ev.reseed
         self.changes_params = False  # set by optimizers: every run rewrites parameter values
 
     def bind(self):
@@ -692,6 +698,8 @@ class Program:
         refresh_derived(self.ctx, self.derived)
         if self.changes_params:
             params_changed()
+        for sx, sy in self.reseed:  # unseeded random fills draw new seeds at every evaluation
+            sx.value, sy.value = fresh_seed()
         for fn, args, _ in self.calls:
             rc = fn(h, *args)
             if rc:
@@ -705,6 +713,9 @@ class Program:
         the constructor, so every expression kernel is built and every buffer exists."""
         if self.graph is not None:
             return self
+        if self.reseed:
+            raise ValueError("a program with unseeded random fills cannot be captured: a graph replays fixed kernel "
+                             "arguments, so every replay would repeat the same random numbers (give the nodes seeds)")
         lib, h = self.ctx._lib, self.ctx.handle
         self.ctx.check(lib.sg_graph_begin(h))
         rc_call = 0
@@ -787,6 +798,8 @@ def _merge_common_subgraphs(targets):
         v.inputs = tuple(canon[id(i)] for i in v.inputs)
         key = (v.op, v.dtype, tuple(v.shape.extents), tuple(v.shape.strides), v.shape.offset,
                repr(sorted(v.attrs.items(), key=lambda kv: kv[0])), tuple(id(i) for i in v.inputs))
+        if v.op in ("rand_uniform", "rand_normal") and v.attrs.get("seed") is None:
+            key += (id(v),)  # every unseeded node is its own draw (rand.rs:70, 113): never merged
         canon[id(v)] = table.setdefault(key, v)
 
 
@@ -820,6 +833,7 @@ class _Evaluator:
         # retained intermediate (recompute time per byte) is dropped and recomputed on demand later.  A
         # recorded Program keeps every buffer instead: its launches are replayed on them.
         self.derived = []  # cached derived-data entries this evaluation relies on (see refresh_derived)
+        self.reseed = []   # seed arguments of unseeded random fills (drawn per evaluation, rand.rs:70, 113)
         self.release = record is None
         self.computed = set()
         self.evictions = 0
@@ -1099,12 +1113,16 @@ class _Evaluator:
 
     def _ev_rand(self, v):
         seed = v.attrs["seed"]
-        if seed is None:
-            seed = tuple(int(b) for b in np.frombuffer(os.urandom(8), np.uint32))
+        fresh = seed is None
+        if fresh:
+            seed = fresh_seed()
         y = self.out(v.extents, FLOAT)
         yc = y.c()
         fn = self.lib.sg_rand_uniform if v.op == "rand_uniform" else self.lib.sg_rand_normal
-        self.call(fn, C.c_uint32(seed[0] & 0xFFFFFFFF), C.c_uint32(seed[1] & 0xFFFFFFFF), C.byref(yc))
+        sx, sy = C.c_uint32(seed[0] & 0xFFFFFFFF), C.c_uint32(seed[1] & 0xFFFFFFFF)
+        self.call(fn, sx, sy, C.byref(yc))
+        if fresh:
+            self.reseed.append((sx, sy))  # a recorded Program redraws these before every replay
         return y
 
     _ev_rand_uniform = _ev_rand_normal = _ev_rand

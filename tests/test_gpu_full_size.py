@@ -101,6 +101,126 @@ def test_config3_bert_layer_b32_s128(ctx, reference_exact):
     close(y, yo, REL_GEMM, "vs oracle")
 
 
+LAYER_KEYS = ["wk", "bk", "wq", "bq", "wv", "bv", "wo", "bo", "ln1_g", "ln1_b", "w1", "b1", "w2", "b2", "ln2_g", "ln2_b"]
+
+
+def oracle_bert_params(arrays, layers, segments):
+    """Host arrays in Bert.params() order -> the oracle's parameter dict."""
+    it = iter(arrays)
+    p = {"word_emb": ht(next(it)), "pos_emb": ht(next(it))}
+    if segments:
+        p["seg_emb"] = ht(next(it))
+    p["emb_g"], p["emb_b"] = ht(next(it)), ht(next(it))
+    p["layers"] = [{k: ht(next(it)) for k in LAYER_KEYS} for _ in range(layers)]
+    p["wc"], p["bc"] = ht(next(it)), ht(next(it))
+    assert next(it, None) is None
+    return p
+
+
+def worst(a, b):
+    """max |a-b| / max(|b|, rms(b)): the figure `close` bounds, as a number to print."""
+    a, b = a.astype(np.float64), b.astype(np.float64)
+    return float(np.max(np.abs(a - b) / np.maximum(np.abs(b), np.sqrt(np.mean(b * b)))))
+
+
+def as_uint(ids):
+    return ht(ids.view(np.uint32))
+
+
+@pytest.mark.parametrize("variant", ["config", "reference"])
+def test_headline_bert_base_b32_s128_twelve_layers_end_to_end(ctx, variant):
+    """The model bench.py times (same builder, same seed): BERT-base, 12 layers, vocab 30522, b32 x s128.
+    Logits and the last encoder output against the oracle's op-for-op evaluation of Bert::pass
+    (bert.rs:72-81, 128-139), within the end-to-end bound of rel 1e-3."""
+    import bench
+    say("headline BERT-base b32 s128, 12 layers, end to end:", variant)
+    d = bench.build_bert(ctx, variant, 32, 128, 12, np.random.default_rng(5), detail=True)
+    prog = S.Program(ctx, [d["logits"], d["hidden"]])
+    logits, hidden = (t.numpy() for t in prog.outputs)
+    say("launches per step", len(prog.calls))
+    exact_variant = variant == "reference"
+    po = oracle_bert_params(d["arrays"], 12, 0 if exact_variant else 2)
+    act, eps, cls = ("relu", 1e-5, 1) if exact_variant else ("gelu", 1e-12, 0)
+    seg = None if d["segment_ids"] is None else as_uint(d["segment_ids"])
+    lo, ho = O.bert_forward(as_uint(d["ids"]), ht(d["mask"]), po, 12, act, eps, cls, seg, return_hidden=True)
+    lo, ho = lo.numpy(), ho.numpy()
+    say(f"worst error / tolerance scale: logits {worst(logits, lo):.3e}, last encoder output {worst(hidden, ho):.3e} (bound 1e-3)")
+    assert logits.shape == (32, 2) and hidden.shape == (32, 128, 768)
+    close(hidden, ho, REL_GEMM, "last encoder output vs oracle")
+    close(logits, lo, REL_GEMM, "logits vs oracle")
+    # the replayed program (what the benchmark times) gives the same bits as its first evaluation
+    prog.run()
+    assert np.array_equal(prog.outputs[0].numpy(), logits)
+
+
+def test_config5_full_bert_base_b64_s512_segments(ctx):
+    """Configuration 5 as written: 12 layers, b64 x s512, vocab 30522, position and segment embeddings,
+    classifier on the [CLS] token.  The oracle cannot run 32768 tokens through 12 layers in seconds, so:
+    the embedding gather at [32768,768] (stride-0 index, layers.rs:430-446) is bit-exact against numpy
+    fancy indexing, the first two sequences of the full batch equal a batch-of-2 run, that run equals the
+    oracle end to end, and everything is finite."""
+    from sage_amd.bert import Bert
+    say("C5 full BERT-base b64 s512 with segment embeddings")
+    rng = np.random.default_rng(55)
+    n, l, layers = 64, 512, 12
+    cfg = BertConfig.base()
+    model = Bert(cfg, reference_exact=False, segments=2)
+    arrays = []
+    for p in model.params():
+        name = p.label or ""
+        if "layer_norm.gamma" in name:
+            a = (1.0 + 0.1 * rng.standard_normal(p.extents)).astype(np.float32)
+        elif "layer_norm.beta" in name or name.endswith(".bias"):
+            a = (0.05 * rng.standard_normal(p.extents)).astype(np.float32)
+        else:
+            a = (rng.standard_normal(p.extents) * 0.02).astype(np.float32)
+        arrays.append(a)
+    load_params(ctx, model, arrays)
+    ids = rng.integers(0, cfg.num_vocabs, (n, l)).astype(np.int32)
+    ids[0, :4] = [0, cfg.num_vocabs - 1, 0, cfg.num_vocabs - 1]  # both ends of the table
+    seg = rng.integers(0, 2, (n, l)).astype(np.int32)
+    mask = np.ones((n, l), np.float32)
+    mask[1, 300:] = 0.0
+    mask[63, 17:] = 0.0
+
+    say("embedding gather [32768,768] from the 30522-row table")
+    we = model.embedding.word_emb.pass_(dev(ctx, ids)).eval(ctx).numpy()
+    assert np.array_equal(we, arrays[0][ids])
+    se = model.embedding.seg_emb.pass_(dev(ctx, seg)).eval(ctx).numpy()
+    assert np.array_equal(se, arrays[2][seg])
+    e_sum = (model.embedding.word_emb.pass_(dev(ctx, ids)) + model.embedding.pos_emb.pass_(dev(ctx, np.arange(l, dtype=np.uint32)))
+             + model.embedding.seg_emb.pass_(dev(ctx, seg))).eval(ctx).numpy()
+    assert np.array_equal(e_sum, (arrays[0][ids] + arrays[1][:l]) + arrays[2][seg])
+
+    def run(sl):
+        ids_v, mask_v, seg_v = dev(ctx, ids[sl]), dev(ctx, mask[sl]), dev(ctx, seg[sl])
+        hidden = model.encode(model.embedding.pass_(ids_v, ctx, seg_v), mask_v)
+        out = V.evaluate_fresh(ctx, [model.classify(hidden), hidden])
+        return out[0].numpy(), out[1].numpy()
+
+    say("full batch")
+    logits_full, hidden_full = run(slice(0, n))
+    assert logits_full.shape == (n, 2) and hidden_full.shape == (n, l, 768)
+    assert np.all(np.isfinite(logits_full)) and np.all(np.isfinite(hidden_full))
+    say("batch of 2 and batch-slice invariance")
+    logits_two, hidden_two = run(slice(0, 2))
+    close(hidden_full[:2], hidden_two, REL_GEMM, "first two sequences of the full batch vs a batch of two")
+    close(logits_full[:2], logits_two, REL_GEMM, "logits, batch-slice invariance")
+    logits_last, hidden_last = run(slice(62, 64))
+    close(hidden_full[62:], hidden_last, REL_GEMM, "last two sequences (one heavily masked)")
+    say("batch of 2 vs the oracle, 12 layers end to end")
+    po = oracle_bert_params(arrays, layers, 2)
+    lo, ho = O.bert_forward(as_uint(ids[:2]), ht(mask[:2]), po, 12, "gelu", 1e-12, 0, as_uint(seg[:2]), return_hidden=True)
+    say(f"worst error / tolerance scale: logits {worst(logits_two, lo.numpy()):.3e}, hidden {worst(hidden_two, ho.numpy()):.3e} (bound 1e-3)")
+    close(hidden_two, ho.numpy(), REL_GEMM, "batch of 2 vs oracle: last encoder output")
+    close(logits_two, lo.numpy(), REL_GEMM, "batch of 2 vs oracle: logits")
+    # every layer ends in a LayerNorm: undoing the last one's affine part leaves rows of mean 0, variance 1
+    g, b = arrays[-4].astype(np.float64), arrays[-3].astype(np.float64)
+    z = (hidden_full.astype(np.float64) - b) / g
+    assert np.abs(z.mean(-1)).max() < 1e-3
+    close(z.var(-1), np.ones(z.shape[:2]), REL_GEMM, "rows normalised")
+
+
 def test_config4_resnet18_b128(ctx):
     say("C4 ResNet-18 b128 28x28x1")
     rng = np.random.default_rng(4)

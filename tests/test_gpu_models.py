@@ -10,7 +10,7 @@ from sage_amd import var as V
 from sage_amd.bert import Bert, BertConfig, BertLayer
 from sage_amd.layers import load_params
 from sage_amd.resnet import ResNet, ResNetConfig
-from tests.util import REL_GEMM, close, exact
+from tests.util import REL_GEMM, REL_MAP, close, exact
 
 pytestmark = pytest.mark.gpu
 
@@ -319,3 +319,41 @@ def test_other_model_families_vs_oracle(ctx, name):
     y2 = model.pass_(dev(ctx, x)).eval(ctx).numpy()
     close(y2, yo, REL_GEMM, "operator by operator vs oracle")
     say("launches", fused, "fused,", ctx.launches - n0, "operator by operator")
+
+
+def test_batch_norm_2d_function_and_layer(ctx):
+    """batch_norm_2d (conv.rs:167-185): gamma * (x - mean) / sqrt(var + eps) + beta with per-channel
+    statistics broadcast over [N,H,W,C]; BatchNorm2d (layers.rs:479-548) normalises with its running
+    statistics, scalar gamma/beta and a hard-coded eps of 1e-05.  Against float64 and the oracle's maps."""
+    from sage_amd.layers import BatchNorm2d
+    say("batch_norm_2d")
+    rng = np.random.default_rng(21)
+    n, h, w, c = 3, 5, 7, 12
+    x = rng.standard_normal((n, h, w, c)).astype(np.float32)
+    mean = rng.standard_normal(c).astype(np.float32)
+    var = rng.uniform(0.2, 3.0, c).astype(np.float32)
+    for gshape in ((1,), (c,)):
+        gamma = rng.uniform(0.5, 1.5, gshape).astype(np.float32)
+        beta = rng.standard_normal(gshape).astype(np.float32)
+        for eps in (1e-5, 0.1):
+            n0 = ctx.launches
+            y = V.batch_norm_2d(dev(ctx, x), dev(ctx, gamma), dev(ctx, beta), dev(ctx, mean), dev(ctx, var), eps).eval(ctx).numpy()
+            assert ctx.launches - n0 == 2  # sqrt(var + eps) on [C], then one fused map over [N,H,W,C]
+            ref = gamma.astype(np.float64) * (x.astype(np.float64) - mean) / np.sqrt(var.astype(np.float64) + np.float32(eps)) + beta
+            close(y, ref, REL_MAP, f"batch_norm_2d gamma{gshape} eps {eps} vs float64")
+            ex = [n, h, w, c]
+            xc = O.binary("div", O.binary("sub", ht(x), ht(mean).expand(ex)), O.unary("sqrt", O.binary("add", ht(var), float(eps))).expand(ex))
+            yo = O.binary("add", O.binary("mul", ht(gamma).expand(ex), xc), ht(beta).expand(ex)).numpy()
+            exact(y, yo, "vs the oracle's maps (+,-,*,/,sqrt are exact)")
+    say("BatchNorm2d layer")
+    layer = BatchNorm2d(c, 0.5)  # the eps given here is ignored by the reference's pass
+    layer.init(ctx, rng)
+    y = layer.pass_(dev(ctx, x)).eval(ctx).numpy()
+    close(y, (x.astype(np.float64) - 1.0) / np.sqrt(1.0 + np.float32(1e-5)) + 1.0, REL_MAP, "initial statistics (all ones)")
+    layer.running_mean.set(S.Tensor.from_numpy(ctx, mean))
+    layer.running_var.set(S.Tensor.from_numpy(ctx, var))
+    layer.gamma.set(S.Tensor.from_numpy(ctx, np.array([1.25], np.float32)))
+    layer.beta.set(S.Tensor.from_numpy(ctx, np.array([-0.5], np.float32)))
+    y = layer.pass_(dev(ctx, x)).eval(ctx).numpy()
+    close(y, 1.25 * (x.astype(np.float64) - mean) / np.sqrt(var.astype(np.float64) + np.float32(1e-5)) - 0.5, REL_MAP, "running statistics")
+    assert [p.label for p in layer.params()] == ["batch_norm_2d.gamma", "batch_norm_2d.beta"]

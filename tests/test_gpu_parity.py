@@ -61,7 +61,7 @@ EXACT_UNARY = {"copy", "abs", "neg", "recip", "sqrt", "square", "sign", "ceil", 
 @pytest.mark.parametrize("shape", [(64, 256), (7, 13), (3, 5, 4)], ids=["vec", "odd", "rank3"])
 def test_unary_maps(ctx, name, shape):
     say("unary", name, shape)
-    rng = np.random.default_rng(hash(name) % 1000)
+    rng = np.random.default_rng(100 + abi.UNARY.index(name))
     lo, hi = UNARY_DOMAIN.get(name, (-3.0, 3.0))
     x = rng.uniform(lo, hi, shape).astype(np.float32)
     if name in ("sign", "ceil", "floor", "round", "abs"):
@@ -432,6 +432,30 @@ def test_gemm_batched_split_k(ctx, monkeypatch):
     y = V.gemm_batched(dev(ctx, a), dev(ctx, b), False, False).eval(ctx).numpy()
     close(y, np.einsum("bmk,bkn->bmn", a.astype(np.float64), b.astype(np.float64)), REL_GEMM, "batched split")
     close(y, O.gemm_batched(ht(a), ht(b), False, False).numpy(), REL_GEMM, "vs oracle")
+
+
+@pytest.mark.parametrize("split", [None, "3"])
+def test_matmul_strided_residual_with_flattened_batch(ctx, monkeypatch, split):
+    """C has two batch axes [2,3,M,N]; the residual is [6,M,N] (batch axes flattened), [2,3,M,N] or a
+    single [M,N]-per-batch view: all three address batch entry b0*3+b1 (straight through the C ABI)."""
+    say("matmul_strided residual layouts", split)
+    if split:
+        monkeypatch.setenv("SAGE_GEMM_SPLITK", split)
+    lib = abi.lib()
+    rng = np.random.default_rng(91)
+    b0, b1, m, k, n = 2, 3, 40, 96, 36
+    a = rng.uniform(-1, 1, (b0, b1, m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (b0, b1, k, n)).astype(np.float32)
+    r = rng.uniform(-1, 1, (b0, b1, m, n)).astype(np.float32)
+    ref = np.einsum("abmk,abkn->abmn", a.astype(np.float64), b.astype(np.float64)) + r
+    ta, tb = S.Tensor.from_numpy(ctx, a), S.Tensor.from_numpy(ctx, b)
+    for res_host in (r.reshape(b0 * b1, m, n), r):
+        tr = S.Tensor.from_numpy(ctx, res_host)
+        out = S.Tensor.uninit(ctx, [b0, b1, m, n])
+        ac, bc, oc, rc_ = ta.c(), tb.c(), out.c(), tr.c()
+        epi = abi.sg_gemm_epilogue(1.0, abi.ACT_NONE, abi.ACT_NONE, None, C.pointer(rc_))
+        ctx.check(lib.sg_matmul_strided(ctx.handle, C.byref(ac), C.byref(bc), C.byref(oc), C.byref(epi)))
+        close(out.numpy(), ref, REL_GEMM, f"residual rank {res_host.ndim}")
 
 
 def test_gemm_offsets_and_ld(ctx):

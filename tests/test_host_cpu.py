@@ -280,3 +280,17 @@ def test_model_families_build_without_a_device():
     w = kaiming_uniform(rng, [64, 256])
     assert w.dtype == np.float32 and np.abs(w).max() <= np.sqrt(3.0 / 256) + 1e-7
     assert abs(float(kaiming_normal(rng, [3, 3, 64, 64]).std()) - np.sqrt(1.0 / (3 * 64 * 64))) < 2e-3
+
+
+def test_unseeded_random_nodes_are_never_merged():
+    """Two unseeded fills are two independent draws (rand.rs:70, 113); seeded ones with the same seed and
+    extents are the same values and may share a node."""
+    from sage_amd import var as V
+    a, b = V.uniform([8]), V.uniform([8])
+    y = a + b
+    V._merge_common_subgraphs([y])
+    assert y.inputs[0] is not y.inputs[1]
+    c, d = V.normal([8], (1, 2)), V.normal([8], (1, 2))
+    z = c + d
+    V._merge_common_subgraphs([z])
+    assert z.inputs[0] is z.inputs[1]

@@ -204,54 +204,50 @@ def cpu_baseline(variant, batch, seq, rng_seed):
 # Single-kernel workloads (the other configurations the parity tests cover).  Each rotates over
 # enough distinct buffer sets to exceed the 256 MB Infinity Cache, so the rate is an HBM rate.
 def kernel_workloads(ctx, name, rng):
-    """name -> (list of call closures to rotate over, algorithmic bytes per call, flops per call,
-    kernel label, oracle thunk for the CPU baseline or None, unit description)."""
+    """name -> (list of programs to rotate over, algorithmic bytes per call, flops per call,
+    kernel label, spec of the oracle's CPU baseline or None).  Every buffer set is a distinct device
+    allocation (so the caches cannot serve the next launch) filled from one host array."""
     import sage_amd as S
-    from sage_amd import abi, nn
-    from sage_amd import var as V
-    lib = abi.lib()
+    from sage_amd import nn
 
     def dev(a):
         return S.Var.new(S.Tensor.from_numpy(ctx, a))
 
     def programs(build, nbuf):
-        progs = [S.Program(ctx, [build(i)]) for i in range(nbuf)]
-        return progs
+        return [S.Program(ctx, [build(i)]) for i in range(nbuf)]
+
+    def normal(*shape):
+        return rng.standard_normal(shape, dtype=np.float32)
 
     if name == "softmax_ce":      # config 1: logits [8192,1024] f32, labels int32 -> loss [8192]
         B, Cn = 8192, 1024
-        nbuf = 20
-        lab = rng.integers(0, Cn, (B, 1)).astype(np.int32)
-        progs = programs(lambda i: nn.softmax_cross_entropy(dev(rng.standard_normal((B, Cn)).astype(np.float32)), dev(lab)), nbuf)
+        lab, x = rng.integers(0, Cn, (B, 1)).astype(np.int32), normal(B, Cn)
+        progs = programs(lambda i: nn.softmax_cross_entropy(dev(x), dev(lab)), 20)
         return progs, B * Cn * 4 + B * 4 + B * 4, 0.0, "softmax_ce_row_kernel<4, 64>", ("softmax_ce", B, Cn)
     if name == "map_exp_sub":     # exp(x0 - x1), x1 broadcast per row (the largest map of config 1)
         B, Cn = 8192, 1024
-        nbuf = 12
-        c = rng.standard_normal((B, 1)).astype(np.float32)
-        progs = programs(lambda i: (dev(rng.standard_normal((B, Cn)).astype(np.float32)) - dev(c)).exp(), nbuf)
+        c, x = normal(B, 1), normal(B, Cn)
+        progs = programs(lambda i: (dev(x) - dev(c)).exp(), 12)
         return progs, 2 * B * Cn * 4 + B * 4, 0.0, "sg_map", ("map_exp_sub", B, Cn)
     if name == "bias_residual":   # (g + bias) + x on [4096, 3072]: 3-input fused map
         M, N = 4096, 3072
-        nbuf = 8
-        bias = rng.standard_normal((N,)).astype(np.float32)
-        progs = programs(lambda i: (dev(rng.standard_normal((M, N)).astype(np.float32)) + dev(bias)) + dev(rng.standard_normal((M, N)).astype(np.float32)), nbuf)
+        bias, g, x = normal(N), normal(M, N), normal(M, N)
+        progs = programs(lambda i: (dev(g) + dev(bias)) + dev(x), 8)
         return progs, 3 * M * N * 4 + N * 4, 0.0, "sg_map", None
     if name == "layer_norm":      # [32768, 768] rows (BERT b64 s512), per-feature gamma/beta
         R, Cn = 32768, 768
-        nbuf = 6
-        g, b = dev(np.ones(Cn, np.float32)), dev(np.zeros(Cn, np.float32))
-        progs = programs(lambda i: nn.layer_norm(dev(rng.standard_normal((R, Cn)).astype(np.float32)), 1, g, b, 1e-12), nbuf)
-        return progs, 2 * R * Cn * 4 + 2 * Cn * 4, 0.0, "layer_norm_row_kernel<3, 64>", None
+        g, b, x = dev(np.ones(Cn, np.float32)), dev(np.zeros(Cn, np.float32)), normal(R, Cn)
+        progs = programs(lambda i: nn.layer_norm(dev(x), 1, g, b, 1e-12), 6)
+        return progs, 2 * R * Cn * 4 + 2 * Cn * 4, 0.0, "layer_norm_row_kernel<3, 64, true>", None
     if name == "softmax":         # attention scores [32,12,128,128] + mask
         n, h, l = 32, 12, 128
-        nbuf = 12
-        m = dev(np.zeros((n, 1, 1, l), np.float32))
-        progs = programs(lambda i: nn.softmax(dev(rng.standard_normal((n, h, l, l)).astype(np.float32)) + m, 3), nbuf)
-        return progs, 2 * n * h * l * l * 4 + n * l * 4, 0.0, "softmax_row_kernel<4, 8, true>", None
+        m, x = dev(np.zeros((n, 1, 1, l), np.float32)), normal(n, h, l, l)
+        progs = programs(lambda i: nn.softmax(dev(x) + m, 3), 12)
+        return progs, 2 * n * h * l * l * 4 + n * l * 4, 0.0, "softmax_row_kernel<4, 8, true, true>", None
     if name == "reduce_sum":      # row sums of [8192,1024]
         B, Cn = 8192, 1024
-        nbuf = 20
-        progs = programs(lambda i: dev(rng.standard_normal((B, Cn)).astype(np.float32)).sum(1, True), nbuf)
+        x = normal(B, Cn)
+        progs = programs(lambda i: dev(x).sum(1, True), 20)
         return progs, B * Cn * 4 + B * 4, 0.0, "reduce_row_kernel<0, float, true, false>", None
     if name == "copy":            # plain copy of 64 Mi floats: the kernel of known size that calibrates FETCH_SIZE / WRITE_SIZE
         n = 64 << 20
@@ -295,13 +291,12 @@ def oracle_kernel_baseline(spec, rng):
     return None, None
 
 
-def run_kernel_workload(a):
-    import sage_amd as S
+def time_kernel_workload(ctx, name, steps, warmup):
+    """Times `steps` launches of one single-kernel workload (after `warmup`) between two HIP events on the
+    context's stream, rotating over its buffer sets.  Returns (roofline dict, config dict, oracle spec)."""
     from sage_amd import abi
     lib = abi.lib()
-    ctx = S.Context(0)
-    rng = np.random.default_rng(1)
-    progs, bytes_per, flops_per, label, spec = kernel_workloads(ctx, a.workload, rng)
+    progs, bytes_per, flops_per, label, spec = kernel_workloads(ctx, name, np.random.default_rng(1))
     launches = len(progs[0].calls)
 
     def ev():
@@ -309,31 +304,58 @@ def run_kernel_workload(a):
         ctx.check(lib.sg_event_create(ctx.handle, C.byref(e)))
         return e
 
-    for i in range(a.warmup):
+    for i in range(warmup):
         progs[i % len(progs)].run()
     ctx.sync()
     e0, e1 = ev(), ev()
     t0 = time.perf_counter()
     lib.sg_event_record(ctx.handle, e0)
-    for i in range(a.steps):
+    for i in range(steps):
         progs[i % len(progs)].run()
     lib.sg_event_record(ctx.handle, e1)
     ctx.sync()
-    dt = time.perf_counter() - t0
+    wall_ms = (time.perf_counter() - t0) / steps * 1e3
     ms = C.c_float()
     ctx.check(lib.sg_event_elapsed_ms(ctx.handle, e0, e1, C.byref(ms)))
-    per_ms = ms.value / a.steps
+    for e in (e0, e1):
+        lib.sg_event_destroy(ctx.handle, e)
+    per_ms = ms.value / steps
     if flops_per:
         achieved, peak, unit, bound = flops_per / (per_ms * 1e-3) / 1e12, PEAK_FP32_MFMA_TFLOPS, "TFLOP/s", "mfma"
     else:
         achieved, peak, unit, bound = bytes_per / (per_ms * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s", "hbm"
-    res = {"metric": f"{a.workload} throughput", "value": achieved, "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-           "ms_per_step": dt / a.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
-           "data": "synthetic",
-           "config": {"workload": a.workload, "launches_per_step": launches, "buffer_sets": len(progs),
-                      "algorithmic_bytes_per_step": bytes_per, "flops_per_step": flops_per},
-           "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
-                        "traffic": measured_traffic(label, a.workload), "kernel": label, "avg_launch_ms": per_ms}}
+    roof = {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
+            "traffic": measured_traffic(label, name), "kernel": label, "avg_launch_ms": per_ms}
+    cfg = {"workload": name, "launches_per_step": launches, "buffer_sets": len(progs),
+           "algorithmic_bytes_per_step": bytes_per, "flops_per_step": flops_per, "wall_ms_per_step": wall_ms}
+    del progs
+    return roof, cfg, spec
+
+
+# The HBM half of the metric: the fused map / reduce / row kernels at the shapes of configurations 1, 3 and 5.
+HBM_WORKLOADS = ("softmax_ce", "reduce_sum", "map_exp_sub", "softmax", "bias_residual", "layer_norm")
+
+
+def hbm_rooflines(ctx, steps=600, warmup=200):
+    """One roofline entry per fused HBM-bound kernel, each timed back to back on rotating buffer sets."""
+    out = []
+    for name in HBM_WORKLOADS:
+        roof, cfg, _ = time_kernel_workload(ctx, name, steps, warmup)
+        out.append({"workload": name, "kernel": roof["kernel"], "bytes": cfg["algorithmic_bytes_per_step"],
+                    "avg_launch_ms": roof["avg_launch_ms"], "achieved": roof["achieved"], "unit": "GB/s",
+                    "frac": roof["frac"], "traffic": roof["traffic"], "launches_timed": steps})
+        ctx.trim()
+    return out
+
+
+def run_kernel_workload(a):
+    import sage_amd as S
+    ctx = S.Context(0)
+    roof, cfg, spec = time_kernel_workload(ctx, a.workload, a.steps, a.warmup)
+    unit, flops_per, bytes_per = roof["unit"], cfg["flops_per_step"], cfg["algorithmic_bytes_per_step"]
+    res = {"metric": f"{a.workload} throughput", "value": roof["achieved"], "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+           "ms_per_step": cfg.pop("wall_ms_per_step"), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+           "data": "synthetic", "config": cfg, "roofline": roof}
     if spec is not None and not a.no_cpu_baseline:
         t, sample = oracle_kernel_baseline(spec, np.random.default_rng(2))
         if t:
@@ -405,8 +427,9 @@ def main():
     ap.add_argument("--seq", type=int, default=128)
     ap.add_argument("--layers", type=int, default=12)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-hbm-kernels", action="store_true", help="bert: leave out the roofline_hbm list (the fused map/reduce/row kernels timed after the model)")
     ap.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
-                    help="replay the step as one HIP graph (auto: on for resnet18, whose step is bound by host launches)")
+                    help="replay the step as one HIP graph (auto = on; off: one host call per operator launch)")
     a = ap.parse_args()
     single_kernel = a.workload not in ("bert", "resnet18", "resnet18_train")
     if a.steps is None:
@@ -458,7 +481,7 @@ def main():
     dom_calls = [i for i, _, _ in by_name[dom]]
     pairs = [{i: (new_event(), new_event()) for j, i in enumerate(dom_calls) if j % SAMPLE == step % SAMPLE} for step in range(a.steps)]
 
-    use_graph = a.graph == "on" or (a.graph == "auto" and a.workload == "resnet18")
+    use_graph = a.graph != "off"
     if use_graph:
         prog.capture()
     for _ in range(a.warmup):
@@ -480,19 +503,21 @@ def main():
             run_timed(ctx, prog, pairs[step])
         ctx.sync()
         dt = time.perf_counter() - t0
-    kernel_ms, kernel_flops = [], []
     flops_of = {i: f for i, f, _ in by_name[dom]}
+    ms_of = {i: [] for i in flops_of}
     for step in range(a.steps):
         for i, (e0, e1) in pairs[step].items():
             ms = C.c_float()
             ctx.check(lib.sg_event_elapsed_ms(ctx.handle, e0, e1, C.byref(ms)))
-            kernel_ms.append(ms.value)
-            kernel_flops.append(flops_of[i])
+            ms_of[i].append(ms.value)
     ms_per_step = dt / a.steps * 1e3
 
-    # the timed launches' own flops over their own time (the sample covers every launch index when steps is a multiple of SAMPLE)
-    flops_per_launch = float(np.mean(kernel_flops))
-    avg_ms = float(np.mean(kernel_ms))
+    # Every launch index of the kernel counts once, whatever number of steps sampled it: the mean duration of
+    # each index first, then flops and time summed over the indices (all of them are sampled when steps >= SAMPLE).
+    sampled = [i for i in ms_of if ms_of[i]]
+    n_timed = sum(len(ms_of[i]) for i in sampled)
+    flops_per_launch = float(np.mean([flops_of[i] for i in sampled]))
+    avg_ms = float(np.mean([np.mean(ms_of[i]) for i in sampled]))
     achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
     total_gemm_flops = sum(f for _, _, f, _ in gc)
     if a.workload == "resnet18":
@@ -516,9 +541,16 @@ def main():
                      "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
                      "traffic": measured_traffic(dom, f"bert_base_b{a.batch}_s{a.seq}") if a.workload == "bert" and a.layers == 12 and a.variant == "config" else None,
                      "kernel": dom,
-                     "launches_per_step": len(by_name[dom]), "launches_timed": len(kernel_ms), "avg_launch_ms": avg_ms, "flops_per_launch": flops_per_launch,
+                     "launches_per_step": len(by_name[dom]), "launch_indices_sampled": len(sampled), "launches_timed": n_timed, "avg_launch_ms": avg_ms, "flops_per_launch": flops_per_launch,
                      "shapes_mnkb": sorted({s for _, _, s in by_name[dom]})},
     }
+    if a.workload == "bert" and not a.no_hbm_kernels:
+        # the other half of the metric: the fused map / reduce / row kernels against the HBM peak
+        if use_graph:
+            prog.release_graph()
+        del prog
+        ctx.trim()
+        res["roofline_hbm"] = hbm_rooflines(ctx)
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline_resnet18(model, arrays, x_host) if a.workload == "resnet18" else cpu_baseline(a.variant, a.batch, a.seq, 6)
     print(json.dumps(res))

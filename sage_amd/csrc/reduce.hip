@@ -60,17 +60,20 @@ struct Dims {
     int n;
     uint32_t ext[SG_MAX_RANK];
     uint32_t stride[SG_MAX_RANK];
+    uint32_t magic[SG_MAX_RANK], shift[SG_MAX_RANK];  // division by ext[a] as a multiply-high and a shift
 };
 
-// linear index over `d.ext` (row-major) -> element offset
+// linear index over `d.ext` (row-major) -> element offset.  No hardware division: ids are below 2^31
+// (checked on the host), where q = (umulhi(id, magic) + id) >> shift is exact; the outermost axis needs
+// no division at all.
 __device__ __forceinline__ uint32_t decompose(const Dims &d, uint32_t id) {
     uint32_t off = 0;
-    for (int a = d.n - 1; a >= 0; --a) {
-        uint32_t q = id / d.ext[a];
+    for (int a = d.n - 1; a > 0; --a) {
+        const uint32_t q = (__umulhi(id, d.magic[a]) + id) >> d.shift[a];
         off += (id - q * d.ext[a]) * d.stride[a];
         id = q;
     }
-    return off;
+    return d.n > 0 ? off + id * d.stride[0] : off;
 }
 
 // ---- one thread per output, nested walk over the reduced axes -------------------------------
@@ -237,12 +240,23 @@ template <int NCHUNK> struct RowRegs {
     f32x4 v[NCHUNK];
 };
 
-template <int NCHUNK, int LPR>
+// NT: non-temporal accesses for rows that stream through (operands too large for the caches to hand
+// them to the next kernel).  Streamed stores also leave the L2s while the kernel runs instead of being
+// written back all at once when it ends.
+template <bool NT> __device__ __forceinline__ f32x4 load4(const float *p) {
+    return NT ? __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p)) : *reinterpret_cast<const f32x4 *>(p);
+}
+template <bool NT> __device__ __forceinline__ void store4(float *p, f32x4 v) {
+    if (NT) __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(p));
+    else *reinterpret_cast<f32x4 *>(p) = v;
+}
+
+template <int NCHUNK, int LPR, bool NT = false>
 __device__ __forceinline__ void load_row(const float *p, uint32_t len, int li, RowRegs<NCHUNK> &r, float fill) {
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
         uint32_t c = (j * LPR + li) * 4u;
-        if (c < len) r.v[j] = *reinterpret_cast<const f32x4 *>(p + c);
+        if (c < len) r.v[j] = load4<NT>(p + c);
         else r.v[j] = f32x4{fill, fill, fill, fill};
     }
 }
@@ -263,7 +277,7 @@ struct BDims {  // broadcastable operand: strides over the row index space + inn
 // max: the reference's max accumulator starts at literal 0 (reduce.rs:282), and using the same
 // shift keeps even the underflow behaviour of rows far below zero identical.  The quotient y/sum is
 // formed as y * (1/sum): one division per row instead of one per element.
-template <int NCHUNK, int LPR, bool HAS_ADD>
+template <int NCHUNK, int LPR, bool HAS_ADD, bool NT>
 __global__ void __launch_bounds__(256) softmax_row_kernel(const float *__restrict__ x, const float *__restrict__ add,
                                                           float *__restrict__ y, uint32_t n_rows, uint32_t len,
                                                           uint32_t x_off, Dims xo, BDims ao, uint32_t y_off) {
@@ -273,40 +287,59 @@ __global__ void __launch_bounds__(256) softmax_row_kernel(const float *__restric
     if (row >= n_rows) return;
     const float *p = x + x_off + decompose(xo, row);
     RowRegs<NCHUNK> r;
-    load_row<NCHUNK, LPR>(p, len, li, r, -__builtin_inff());
+    load_row<NCHUNK, LPR, NT>(p, len, li, r, -__builtin_inff());
     if (HAS_ADD) {
+        // the addend (a mask broadcast over heads and queries) is re-read by many rows: regular loads
         const float *a = add + ao.off + decompose(ao.outer, row);
+        f32x4 av[NCHUNK];
 #pragma unroll
         for (int j = 0; j < NCHUNK; ++j) {
-            uint32_t c = (j * LPR + li) * 4u;
+            const uint32_t c = (j * LPR + li) * 4u;
+            av[j] = f32x4{0.f, 0.f, 0.f, 0.f};
             if (c < len) {
                 if (ao.inner_stride == 1) {
-                    r.v[j] += *reinterpret_cast<const f32x4 *>(a + c);
+                    av[j] = *reinterpret_cast<const f32x4 *>(a + c);
                 } else {
-                    r.v[j].x += a[(c + 0) * ao.inner_stride]; r.v[j].y += a[(c + 1) * ao.inner_stride];
-                    r.v[j].z += a[(c + 2) * ao.inner_stride]; r.v[j].w += a[(c + 3) * ao.inner_stride];
+                    av[j].x = a[(c + 0) * ao.inner_stride]; av[j].y = a[(c + 1) * ao.inner_stride];
+                    av[j].z = a[(c + 2) * ao.inner_stride]; av[j].w = a[(c + 3) * ao.inner_stride];
                 }
             }
         }
+#pragma unroll
+        for (int j = 0; j < NCHUNK; ++j) r.v[j] += av[j];
     }
     float m = -__builtin_inff();
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) m = fmaxf(fmaxf(fmaxf(fmaxf(m, r.v[j].x), r.v[j].y), r.v[j].z), r.v[j].w);
     m = fmaxf(seg_reduce<OP_MAX, LPR>(m), 0.0f);
+    RowRegs<NCHUNK> e;
     float s = 0.0f;
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
-        r.v[j].x = expf(r.v[j].x - m); r.v[j].y = expf(r.v[j].y - m);
-        r.v[j].z = expf(r.v[j].z - m); r.v[j].w = expf(r.v[j].w - m);
-        s += (r.v[j].x + r.v[j].y) + (r.v[j].z + r.v[j].w);
+        e.v[j].x = fast_exp(r.v[j].x - m); e.v[j].y = fast_exp(r.v[j].y - m);
+        e.v[j].z = fast_exp(r.v[j].z - m); e.v[j].w = fast_exp(r.v[j].w - m);
+        s += (e.v[j].x + e.v[j].y) + (e.v[j].z + e.v[j].w);
     }
     s = seg_reduce<OP_SUM, LPR>(s);
+    // fast_exp flushes results below 2^-126 to zero, which only matters when every term of the row is
+    // that small (a row entirely below -87, whose shift is 0): such a row is redone with the exact
+    // routine, which keeps the denormal terms as the reference's kernel language does
+    if (s < 1.0e-30f) {
+        s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NCHUNK; ++j) {
+            e.v[j].x = expf(r.v[j].x - m); e.v[j].y = expf(r.v[j].y - m);
+            e.v[j].z = expf(r.v[j].z - m); e.v[j].w = expf(r.v[j].w - m);
+            s += (e.v[j].x + e.v[j].y) + (e.v[j].z + e.v[j].w);
+        }
+        s = seg_reduce<OP_SUM, LPR>(s);
+    }
     const float inv = 1.0f / s;
     float *q = y + y_off + (size_t)row * len;
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
         uint32_t c = (j * LPR + li) * 4u;
-        if (c < len) *reinterpret_cast<f32x4 *>(q + c) = r.v[j] * inv;
+        if (c < len) store4<NT>(q + c, e.v[j] * inv);
     }
 }
 
@@ -417,21 +450,21 @@ __global__ void __launch_bounds__(256) softmax_ce_row_generic_kernel(const float
 // y = (x - mean) / sqrt(var + eps) * gamma + beta.  The division by sqrt(var+eps) is applied as a
 // multiplication by its reciprocal (one division per row); everything else keeps the reference's
 // operation order.
-template <int NCHUNK, int LPR>
+template <int NCHUNK, int LPR, bool NT>
 __global__ void __launch_bounds__(256) layer_norm_row_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
                                                              const float *__restrict__ beta, float *__restrict__ y,
                                                              uint32_t n_rows, uint32_t len, uint32_t x_off, Dims xo,
                                                              uint32_t g_off, uint32_t g_stride, uint32_t b_off, uint32_t b_stride,
-                                                             float eps, uint32_t y_off) {
+                                                             int params_aligned, float eps, uint32_t y_off) {
     constexpr int RPW = WAVE / LPR;
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, li = lane % LPR;
     const uint32_t row = (blockIdx.x * 4u + wave) * RPW + lane / LPR;
     if (row >= n_rows) return;
     const float *p = x + x_off + decompose(xo, row);
     RowRegs<NCHUNK> r;
-    load_row<NCHUNK, LPR>(p, len, li, r, 0.0f);
+    load_row<NCHUNK, LPR, NT>(p, len, li, r, 0.0f);
     // gamma and beta are requested with the row, so nothing waits on memory after the statistics
-    const bool vec_params = g_stride == 1 && b_stride == 1 && ((g_off | b_off) & 3u) == 0;
+    const bool vec_params = g_stride == 1 && b_stride == 1 && params_aligned;
     f32x4 gv[NCHUNK], bv[NCHUNK];
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
@@ -466,7 +499,7 @@ __global__ void __launch_bounds__(256) layer_norm_row_kernel(const float *__rest
 #pragma unroll
     for (int j = 0; j < NCHUNK; ++j) {
         const uint32_t c = (j * LPR + li) * 4u;
-        if (c < len) *reinterpret_cast<f32x4 *>(q + c) = (r.v[j] - mean) * inv * gv[j] + bv[j];
+        if (c < len) store4<NT>(q + c, (r.v[j] - mean) * inv * gv[j] + bv[j]);
     }
 }
 
@@ -527,6 +560,9 @@ Dims to_dims(const std::vector<int64_t> &ext, const std::vector<int64_t> &st) {
     for (int i = 0; i < SG_MAX_RANK; ++i) {
         d.ext[i] = i < d.n ? (uint32_t)ext[i] : 1;
         d.stride[i] = i < d.n ? (uint32_t)st[i] : 0;
+        const sg_fastdiv f = sg_make_fastdiv(d.ext[i]);
+        d.magic[i] = f.magic;
+        d.shift[i] = f.shift;
     }
     return d;
 }
@@ -571,9 +607,7 @@ int launch_reduce(sg_ctx *ctx, const sg_tensor *in, const sg_tensor *out, const 
         if (rc != SG_OK) return rc;
         hipLaunchKernelGGL((reduce_cols_kernel<OP, T>), dim3(col_tiles, chunks), dim3(256), 0, ctx->stream, x, (T *)ws, n_cols, n_rows,
                            red.stride[0], rows_per_chunk, (uint32_t)in->offset);
-        Dims pk = kept, pr = red;
-        pr.ext[0] = chunks;
-        pr.stride[0] = n_cols;
+        const Dims pk = kept, pr = to_dims({(int64_t)chunks}, {(int64_t)n_cols});
         hipLaunchKernelGGL((reduce_thread_kernel<OP, T>), dim3((n_cols + 255) / 256), dim3(256), 0, ctx->stream, (const T *)ws, y, n_cols, 0u, pk, pr, chunks, ref_zero);
         SG_CHECK_LAUNCH(ctx, "reduce (columns)");
         return sg_free(ctx, ws);  // later users of the block are ordered behind these kernels on the stream
@@ -734,28 +768,33 @@ extern "C" int sg_softmax_lastaxis(sg_ctx *ctx, const sg_tensor *x, const sg_ten
     const int64_t n_rows = row_dims(x, xo);
     BDims ao{};
     if (addend) {
-        // rows of the addend are indexed with x's row id, so decompose over x's outer extents
+        // Both operands decompose the same row id over the same outer extents, so each may merge its own
+        // adjacent axes wherever ITS strides allow (stride[i] == stride[i+1] * ext[i+1], which a run of
+        // broadcast axes satisfies with zeros): a mask [N,1,1,L] under scores [N,H,L,L] becomes [N, H*L]
+        // with strides [L, 0], one multiply-high per row, and dense scores collapse to a single axis.
         std::vector<int64_t> e(x->extents, x->extents + r - 1), s(addend->strides, addend->strides + r - 1);
-        // no collapse against x's strides here: keep axes as they are so both share the row id
+        collapse(e, s);
         ao.outer = to_dims(e, s);
         ao.inner_stride = (uint32_t)addend->strides[r - 1];
         ao.off = (uint32_t)addend->offset;
-        std::vector<int64_t> xs(x->strides, x->strides + r - 1);
-        xo = to_dims(e, xs);
     }
     const float *xp = (const float *)x->base, *ap = addend ? (const float *)addend->base : nullptr;
     float *yp = (float *)out->base;
     const bool vec = len % 4 == 0 && len <= 2048 && aligned16(x->base, x->offset) && dims_mult4(xo) && aligned16(out->base, out->offset) &&
                      (!addend || ao.inner_stride != 1 || (aligned16(addend->base, addend->offset) && dims_mult4(ao.outer)));
     if (vec) {
+        const bool nt = sg_streaming(2 * sg_numel(x) * 4);
+#define SG_ROW_LAUNCH_(NC, LPR, ADD, NT)                                                                                \
+    hipLaunchKernelGGL((softmax_row_kernel<NC, LPR, ADD, NT>), grid, dim3(256), 0, ctx->stream, xp, ap, yp, (uint32_t)n_rows, len, (uint32_t)x->offset, xo, ao, (uint32_t)out->offset)
 #define SG_ROW_LAUNCH(NC, LPR)                                                                                          \
     do {                                                                                                                \
         dim3 grid((unsigned)((n_rows + 4 * (64 / LPR) - 1) / (4 * (64 / LPR))));                                        \
-        if (addend) hipLaunchKernelGGL((softmax_row_kernel<NC, LPR, true>), grid, dim3(256), 0, ctx->stream, xp, ap, yp, (uint32_t)n_rows, len, (uint32_t)x->offset, xo, ao, (uint32_t)out->offset); \
-        else hipLaunchKernelGGL((softmax_row_kernel<NC, LPR, false>), grid, dim3(256), 0, ctx->stream, xp, ap, yp, (uint32_t)n_rows, len, (uint32_t)x->offset, xo, ao, (uint32_t)out->offset); \
+        if (addend) { if (nt) SG_ROW_LAUNCH_(NC, LPR, true, true); else SG_ROW_LAUNCH_(NC, LPR, true, false); }          \
+        else { if (nt) SG_ROW_LAUNCH_(NC, LPR, false, true); else SG_ROW_LAUNCH_(NC, LPR, false, false); }                \
     } while (0)
         SG_ROW_DISPATCH(len);
 #undef SG_ROW_LAUNCH
+#undef SG_ROW_LAUNCH_
     } else {
         if (addend) hipLaunchKernelGGL((softmax_row_generic_kernel<true>), dim3((unsigned)n_rows), dim3(256), 0, ctx->stream, xp, ap, yp, len, (uint32_t)x->offset, xo, ao, (uint32_t)out->offset);
         else hipLaunchKernelGGL((softmax_row_generic_kernel<false>), dim3((unsigned)n_rows), dim3(256), 0, ctx->stream, xp, ap, yp, len, (uint32_t)x->offset, xo, ao, (uint32_t)out->offset);
@@ -822,13 +861,19 @@ extern "C" int sg_layer_norm_lastaxis(sg_ctx *ctx, const sg_tensor *x, const sg_
     const uint32_t gs = ng == 1 ? 0u : 1u, bs = nb == 1 ? 0u : 1u;
     const bool vec = len % 4 == 0 && len <= 2048 && aligned16(x->base, x->offset) && dims_mult4(xo) && aligned16(out->base, out->offset);
     if (vec) {
+        const bool nt = sg_streaming(2 * sg_numel(x) * 4);
+        // 16-byte loads of gamma and beta need their first elements 16-byte aligned, not just x's
+        const int params_aligned = aligned16(gamma->base, gamma->offset) && aligned16(beta->base, beta->offset);
+#define SG_ROW_LAUNCH_(NC, LPR, NT)                                                                                     \
+    hipLaunchKernelGGL((layer_norm_row_kernel<NC, LPR, NT>), grid, dim3(256), 0, ctx->stream, xp, gp, bp, yp, (uint32_t)n_rows, len, (uint32_t)x->offset, xo, (uint32_t)gamma->offset, gs, (uint32_t)beta->offset, bs, params_aligned, eps, (uint32_t)out->offset)
 #define SG_ROW_LAUNCH(NC, LPR)                                                                                          \
     do {                                                                                                                \
         dim3 grid((unsigned)((n_rows + 4 * (64 / LPR) - 1) / (4 * (64 / LPR))));                                        \
-        hipLaunchKernelGGL((layer_norm_row_kernel<NC, LPR>), grid, dim3(256), 0, ctx->stream, xp, gp, bp, yp, (uint32_t)n_rows, len, (uint32_t)x->offset, xo, (uint32_t)gamma->offset, gs, (uint32_t)beta->offset, bs, eps, (uint32_t)out->offset); \
+        if (nt) SG_ROW_LAUNCH_(NC, LPR, true); else SG_ROW_LAUNCH_(NC, LPR, false);                                     \
     } while (0)
         SG_ROW_DISPATCH(len);
 #undef SG_ROW_LAUNCH
+#undef SG_ROW_LAUNCH_
     } else {
         hipLaunchKernelGGL(layer_norm_row_generic_kernel, dim3((unsigned)n_rows), dim3(256), 0, ctx->stream, xp, gp, bp, yp, len, (uint32_t)x->offset, xo,
                            (uint32_t)gamma->offset, gs, (uint32_t)beta->offset, bs, eps, (uint32_t)out->offset);

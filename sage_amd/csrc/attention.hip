@@ -25,15 +25,15 @@
 // rounding level (covered by the 1e-3 tolerance of GEMM-bearing paths).
 #include "common.h"
 
+#include <cstdlib>
+
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int NW = 4;          // wavefronts per workgroup
-constexpr int QB = 32 * NW;    // queries per workgroup
 constexpr int KB = 64;         // keys per LDS block
-constexpr int NKB = KB / 32;   // 32-key MFMA blocks per LDS block
 
 struct AttnP {
     const float *q, *k, *v, *add;
@@ -45,14 +45,24 @@ struct AttnP {
     int vec_q, vec_k, vec_v, vec_o;
 };
 
-template <int D>
+// SPLIT = false: the four wavefronts take four groups of 32 queries and every wavefront walks all keys.
+// SPLIT = true: the workgroup covers 64 queries; wavefronts 0,1 take the first 32 keys of every 64-key
+// block and wavefronts 2,3 the other 32, and the two partial results of a query group are merged
+// through LDS at the end (the exact merge of two online-softmax states).  Work units are half as
+// large, which is what balances a short-sequence launch: B*H*L/32 units of 32 queries x all keys
+// may come to 1.5 per SIMD (b32, 12 heads, s128: 1536 units on 1024 SIMDs), i.e. two rounds with half
+// the chip idle in the second; split in two they are 3 per SIMD.
+template <int D, bool SPLIT>
 __global__ void __launch_bounds__(64 * NW) attention_kernel(const AttnP p) {
     static_assert(D % 32 == 0 && D <= 64, "head size 32 or 64");
+    constexpr int QB = SPLIT ? 64 : 32 * NW;   // queries per workgroup
+    constexpr int NKB = SPLIT ? 1 : KB / 32;   // 32-key MFMA blocks a wavefront takes from an LDS block
     constexpr int LD = D + 4;              // LDS row stride (floats): 8 consecutive rows cover all banks
     constexpr int ND = D / 32;             // 32-wide blocks of the head dimension
     constexpr int NG = D / 8;              // groups of four k-steps over the head dimension
     constexpr int ROWV = D / 4;            // 16-byte pieces per K/V row
     constexpr int NLD = KB * ROWV / (64 * NW);  // 16-byte pieces of a K (or V) block per thread
+    typedef float vecND __attribute__((ext_vector_type(ND)));  // one V value per output block of the head dimension
     __shared__ __attribute__((aligned(16))) float lds_k[KB * LD];
     __shared__ __attribute__((aligned(16))) float lds_v[KB * LD];
     __shared__ __attribute__((aligned(16))) float lds_m[KB];
@@ -60,7 +70,8 @@ __global__ void __launch_bounds__(64 * NW) attention_kernel(const AttnP p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ql = lane & 31, h = lane >> 5;
     const int bt0 = blockIdx.y / p.nb1, bt1 = blockIdx.y % p.nb1;
-    const int q0 = blockIdx.x * QB + wave * 32;
+    const int q0 = blockIdx.x * QB + (SPLIT ? (wave & 1) : wave) * 32;
+    const int kw = SPLIT ? (wave >> 1) * 32 : 0;  // this wavefront's first key inside an LDS block
     const float *Q = p.q + bt0 * p.q_sb0 + bt1 * p.q_sb1;
     const float *K = p.k + bt0 * p.k_sb0 + bt1 * p.k_sb1;
     const float *V = p.v + bt0 * p.v_sb0 + bt1 * p.v_sb1;
@@ -142,7 +153,7 @@ __global__ void __launch_bounds__(64 * NW) attention_kernel(const AttnP p) {
         for (int g = 0; g < NG; ++g) {
             f32x4 a[NKB];
 #pragma unroll
-            for (int b = 0; b < NKB; ++b) a[b] = *reinterpret_cast<const f32x4 *>(&lds_k[(b * 32 + ql) * LD + 8 * g + 4 * h]);
+            for (int b = 0; b < NKB; ++b) a[b] = *reinterpret_cast<const f32x4 *>(&lds_k[(kw + b * 32 + ql) * LD + 8 * g + 4 * h]);
 #pragma unroll
             for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -155,7 +166,7 @@ __global__ void __launch_bounds__(64 * NW) attention_kernel(const AttnP p) {
         for (int b = 0; b < NKB; ++b)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const f32x4 mk = *reinterpret_cast<const f32x4 *>(&lds_m[b * 32 + 8 * g + 4 * h]);
+                const f32x4 mk = *reinterpret_cast<const f32x4 *>(&lds_m[kw + b * 32 + 8 * g + 4 * h]);
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
                     const float x = sacc[b][4 * g + s] * p.scale + mk[s];
@@ -168,8 +179,17 @@ __global__ void __launch_bounds__(64 * NW) attention_kernel(const AttnP p) {
         // exp(x - m) as 2^(x*log2(e) - m*log2(e)): one fused multiply-add and the hardware exp2; the argument
         // rounding costs about |x - m| * 6e-8 relative, far inside the softmax tolerance
         constexpr float LOG2E = 1.44269504088896340736f;
-        const float corr = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
         const float mshift = -m_new * LOG2E;
+        // the shift rarely moves after the first blocks: when it stayed put for every query of the wavefront the
+        // correction factor is exactly 1 and rescaling the accumulators (vector work the matrix pipe waits for) is skipped
+        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+            const float corr = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
+            l_run *= corr;
+#pragma unroll
+            for (int j = 0; j < ND; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[j][r] *= corr;
+        }
         m_run = m_new;
         float lsum = 0.0f;
 #pragma unroll
@@ -180,44 +200,75 @@ __global__ void __launch_bounds__(64 * NW) attention_kernel(const AttnP p) {
                 sacc[b][r] = e;
                 lsum += e;
             }
-        l_run = l_run * corr + lsum;
-#pragma unroll
-        for (int j = 0; j < ND; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[j][r] *= corr;
+        l_run += lsum;
 
-        // ---- O^T += V^T . P^T: rows = head dimension, columns = queries, contraction over keys
+        // ---- O^T += V^T . P^T: rows = head dimension, columns = queries, contraction over keys.
+        // Row m of output block j stands for head index ND*m + j (any assignment of head indices to rows
+        // works as long as the write-out agrees), so the ND values a lane feeds to the ND blocks for one
+        // key are adjacent in the V row and come out of LDS as ONE read of 4*ND bytes.
 #pragma unroll
         for (int b = 0; b < NKB; ++b)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                float a[ND][4];
+                vecND a[4];
 #pragma unroll
-                for (int j = 0; j < ND; ++j)
-#pragma unroll
-                    for (int s = 0; s < 4; ++s) a[j][s] = lds_v[(b * 32 + 8 * g + 4 * h + s) * LD + j * 32 + ql];
+                for (int s = 0; s < 4; ++s) a[s] = *reinterpret_cast<const vecND *>(&lds_v[(kw + b * 32 + 8 * g + 4 * h + s) * LD + ND * ql]);
 #pragma unroll
                 for (int s = 0; s < 4; ++s)
 #pragma unroll
-                    for (int j = 0; j < ND; ++j) oacc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][s], sacc[b][4 * g + s], oacc[j], 0, 0, 0);
+                    for (int j = 0; j < ND; ++j) oacc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s][j], sacc[b][4 * g + s], oacc[j], 0, 0, 0);
             }
     }
 
-    // ---- normalise and write: register r = 4g + s of block j is head index 32j + 8g + 4h + s
+    if (SPLIT) {
+        // merge the two key halves of a query group: (m, l, O) of wavefront w + 2 into wavefront w, with
+        // m = max(m_a, m_b), l = l_a e^(m_a - m) + l_b e^(m_b - m), O likewise; the K block's LDS is free now
+        constexpr float LOG2E = 1.44269504088896340736f;
+        constexpr int SLOT = 16 * ND + 2;  // floats per lane
+        static_assert(2 * 64 * SLOT <= KB * LD, "the merge buffer fits in the K block");
+        __syncthreads();
+        if (wave >= 2) {
+            float *dst = &lds_k[((wave - 2) * 64 + lane) * SLOT];
+#pragma unroll
+            for (int j = 0; j < ND; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) dst[16 * j + r] = oacc[j][r];
+            dst[16 * ND] = m_run;
+            dst[16 * ND + 1] = l_run;
+        }
+        __syncthreads();
+        if (wave >= 2) return;
+        const float *src = &lds_k[(wave * 64 + lane) * SLOT];
+        const float m_b = src[16 * ND], l_b = src[16 * ND + 1];
+        const float m = fmaxf(m_run, m_b);
+        const float ca = __builtin_amdgcn_exp2f((m_run - m) * LOG2E), cb = __builtin_amdgcn_exp2f((m_b - m) * LOG2E);
+        l_run = l_run * ca + l_b * cb;
+#pragma unroll
+        for (int j = 0; j < ND; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[j][r] = oacc[j][r] * ca + src[16 * j + r] * cb;
+    }
+    // ---- normalise and write: register r = 4g + s of block j is head index ND*(8g + 4h + s) + j, so the
+    // 4*ND values of one g are consecutive head indices starting at ND*(8g + 4h)
     const float l = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = 1.0f / l;
     const int q = q0 + ql;
     if (q < p.Lq) {
         float *row = p.o + bt0 * p.o_sb0 + bt1 * p.o_sb1 + (int64_t)q * p.o_sl;
 #pragma unroll
-        for (int j = 0; j < ND; ++j)
+        for (int g = 0; g < 4; ++g) {
+            float t[4 * ND];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                f32x4 t = {oacc[j][4 * g] * inv, oacc[j][4 * g + 1] * inv, oacc[j][4 * g + 2] * inv, oacc[j][4 * g + 3] * inv};
-                float *dst = row + 32 * j + 8 * g + 4 * h;
-                if (p.vec_o) *reinterpret_cast<f32x4 *>(dst) = t;
-                else { dst[0] = t.x; dst[1] = t.y; dst[2] = t.z; dst[3] = t.w; }
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int j = 0; j < ND; ++j) t[ND * s + j] = oacc[j][4 * g + s] * inv;
+            float *dst = row + ND * (8 * g + 4 * h);
+#pragma unroll
+            for (int c = 0; c < ND; ++c) {
+                if (p.vec_o) *reinterpret_cast<f32x4 *>(dst + 4 * c) = f32x4{t[4 * c], t[4 * c + 1], t[4 * c + 2], t[4 * c + 3]};
+                else { dst[4 * c] = t[4 * c]; dst[4 * c + 1] = t[4 * c + 1]; dst[4 * c + 2] = t[4 * c + 2]; dst[4 * c + 3] = t[4 * c + 3]; }
             }
+        }
     }
 }
 
@@ -285,9 +336,23 @@ extern "C" int sg_attention(sg_ctx *ctx, const sg_tensor *q, const sg_tensor *k,
     p.Lq = (int)Lq; p.Lk = (int)Lk; p.nb1 = (int)nb1;
     p.scale = scale;
     if (nb0 * nb1 > 65535) return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention: more than 65535 (batch x head) pairs");
-    dim3 grid((unsigned)((Lq + QB - 1) / QB), (unsigned)(nb0 * nb1));
-    if (D == 64) hipLaunchKernelGGL((attention_kernel<64>), grid, dim3(64 * NW), 0, ctx->stream, p);
-    else hipLaunchKernelGGL((attention_kernel<32>), grid, dim3(64 * NW), 0, ctx->stream, p);
+    // Few workgroups of 128 queries (less than two per compute unit): halving the work units (see the kernel)
+    // balances the SIMDs, at the price of a later start of a compute unit's third workgroup and the merge.
+    // Measured at b32 x 12 heads: 68 against 76 us at 128 x 512 (queries x keys), 39 against 43 at 128 x 256,
+    // 15 against 22 at 64 x 128, equal at 128 x 128, slower when the chip is full anyway.
+    const int64_t wgs128 = nb0 * nb1 * ((Lq + 127) / 128);
+    const int64_t tail = Lq % 128;
+    bool split = wgs128 < 2 * (int64_t)(ctx->num_cus > 0 ? ctx->num_cus : 256) && (Lk >= 256 || (tail >= 1 && tail <= 64));
+    if (const char *e = getenv("SAGE_ATTENTION_SPLIT")) split = atoi(e) != 0;
+    const int qb = split ? 64 : 128;
+    dim3 grid((unsigned)((Lq + qb - 1) / qb), (unsigned)(nb0 * nb1));
+    if (D == 64) {
+        if (split) hipLaunchKernelGGL((attention_kernel<64, true>), grid, dim3(64 * NW), 0, ctx->stream, p);
+        else hipLaunchKernelGGL((attention_kernel<64, false>), grid, dim3(64 * NW), 0, ctx->stream, p);
+    } else {
+        if (split) hipLaunchKernelGGL((attention_kernel<32, true>), grid, dim3(64 * NW), 0, ctx->stream, p);
+        else hipLaunchKernelGGL((attention_kernel<32, false>), grid, dim3(64 * NW), 0, ctx->stream, p);
+    }
     SG_CHECK_LAUNCH(ctx, "attention");
     return SG_OK;
 }

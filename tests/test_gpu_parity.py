@@ -677,6 +677,33 @@ def test_attention_fused_vs_composed_vs_oracle(ctx, n, h, lq, lk, d, masked):
     assert fused_launches == (2 if masked else 1), fused_launches  # the mask expression + the attention kernel
 
 
+@pytest.mark.parametrize("split", ["0", "1"])
+@pytest.mark.parametrize("n,h,lq,lk,d", [(2, 3, 128, 128, 64), (1, 2, 70, 200, 64), (2, 2, 33, 31, 32), (1, 1, 64, 300, 64)])
+def test_attention_key_split_variant_matches(ctx, monkeypatch, split, n, h, lq, lk, d):
+    """The kernel that gives the two 32-key halves of every key block to different wavefronts and merges their
+    online-softmax states, forced on and off: both agree with float64 attention (ragged key counts leave one half
+    partly or wholly past the end)."""
+    say("attention key split", split, (n, h, lq, lk, d))
+    monkeypatch.setenv("SAGE_ATTENTION_SPLIT", split)
+    lib = abi.lib()
+    rng = np.random.default_rng(lq * 7 + lk)
+    q, k, v = (rng.standard_normal((n, h, l, d)).astype(np.float32) for l in (lq, lk, lk))
+    mask = (rng.uniform(size=(n, 1, 1, lk)) < 0.8).astype(np.float32)
+    add = ((1.0 - mask) * -1e5).astype(np.float32)
+    tq, tk, tv, ta = (S.Tensor.from_numpy(ctx, a) for a in (q, k, v, add))
+    out = S.Tensor.uninit(ctx, [n, h, lq, d])
+    from sage_amd.shape import Shape
+    tadd = ta.with_shape(Shape([n, h, lq, lk], [lk, 0, 0, 1], 0))
+    qc, kc, vc, ac, oc = tq.c(), tk.c(), tv.c(), tadd.c(), out.c()
+    scale = 1.0 / np.sqrt(np.float32(d))
+    ctx.check(lib.sg_attention(ctx.handle, C.byref(qc), C.byref(kc), C.byref(vc), C.byref(ac), C.c_float(scale), C.byref(oc)))
+    s = np.einsum("nhqd,nhkd->nhqk", q.astype(np.float64), k.astype(np.float64)) * float(scale) + add
+    s -= np.maximum(s.max(-1, keepdims=True), 0.0)
+    p_ = np.exp(s)
+    ref = np.einsum("nhqk,nhkd->nhqd", p_ / p_.sum(-1, keepdims=True), v.astype(np.float64))
+    close(out.numpy(), ref, REL_GEMM, "attention vs float64")
+
+
 def test_attention_fully_masked_row_is_reference_nan(ctx):
     """Every key masked by -1e5: the reference's softmax shifts by max(0, row max) = 0, every exp underflows
     and the row is 0/0.  The fused kernel keeps that behaviour instead of a uniform row."""

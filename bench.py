@@ -134,6 +134,13 @@ def gemm_calls(ctx, prog):
     lib = abi.lib()
     out = []
     for i, (fn, args, _) in enumerate(prog.calls):
+        if fn is lib.sg_conv2d:  # the product of the never-written column matrix [N*OH*OW, KH*KW*C] with the filter [KH*KW*C, OC]
+            x, f, c = (a._obj for a in args[:3])
+            M, N, K = c.extents[0] * c.extents[1] * c.extents[2], c.extents[3], f.extents[0] * f.extents[1] * f.extents[2]
+            buf = C.create_string_buffer(128)
+            ctx.check(lib.sg_gemm_kernel_name(ctx.handle, M, N, K, 1, 1, 1, buf, 128))
+            out.append((i, buf.value.decode().replace(">", ", true>").replace("false, true>", "true, true>"), 2.0 * M * N * K + M * N, (M, N, K, 1)))
+            continue
         if fn in (lib.sg_gemm, lib.sg_gemm_batched, lib.sg_matmul_strided):
             if fn is lib.sg_matmul_strided:
                 a, b, c = (x._obj for x in args[:3])

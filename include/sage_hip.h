@@ -254,6 +254,22 @@ int sg_gemm_kernel_name(sg_ctx *ctx, int64_t M, int64_t N, int64_t K, int64_t ba
 int sg_im2col(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, const int32_t ker[2],
               const int32_t stride[2], const int32_t pad[2], const int32_t dil[2]);
 
+/* conv_2d (conv.rs:61-96) in one launch: out[N,OH,OW,OC] = im2col(x)[N*OH*OW, KH*KW*C] . filter[KH*KW*C, OC]
+ * with the column matrix never written (the reference launches Im2col::compute, conv.rs:289-374, and then
+ * Gemm::compute_direct on its output).  x [N,H,W,C], filter [KH,KW,C,OC], out dense; pairs are {w, h};
+ * the kernel size comes from the filter.  epi as in sg_gemm (bias over OC, residual as [N*OH*OW, OC]:
+ * the output seen as a matrix).  A few-tile/long-K product uses a split-K workspace from the context allocator (SG_ERR_OOM). */
+int sg_conv2d(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *filter, const sg_tensor *out,
+              const int32_t stride[2], const int32_t pad[2], const int32_t dil[2],
+              const sg_gemm_epilogue *epi);
+
+/* max_pool_2d / avg_pool_2d (conv.rs:143-165) without the column tensor: out[N,OH,OW,C] = reduce over the
+ * kernel window of x[N,H,W,C], exactly what Im2col::compute (conv.rs:289-374) followed by
+ * ReduceOperator::compute over axes [3,4] (reduce.rs:258-325) gives: pixels outside the image count as
+ * zeros, op and init_mode as in sg_reduce (avg_pool divides the SUM by the window size afterwards). */
+int sg_pool2d(sg_ctx *ctx, int op, int init_mode, const sg_tensor *x, const sg_tensor *out,
+              const int32_t ker[2], const int32_t stride[2], const int32_t pad[2], const int32_t dil[2]);
+
 /* Col2im::compute (conv.rs:405-500), the adjoint of sg_im2col used by Im2col::grad (conv.rs:275-287):
  * x [N,OH,OW,KH,KW,C] dense -> out [N,H,W,C], each pixel the sum of the column entries taken from
  * it (additions in the reference's order: column x outer, column y inner). */

@@ -87,6 +87,8 @@ PROTOTYPES = {
     "sg_matmul_strided": (C.c_int, [_CTX, _TP, _TP, _TP, C.POINTER(sg_gemm_epilogue)]),
     "sg_gemm_kernel_name": (C.c_int, [_CTX, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_char_p, C.c_uint64]),
     "sg_im2col": (C.c_int, [_CTX, _TP, _TP, _I32P, _I32P, _I32P, _I32P]),
+    "sg_conv2d": (C.c_int, [_CTX, _TP, _TP, _TP, _I32P, _I32P, _I32P, C.POINTER(sg_gemm_epilogue)]),
+    "sg_pool2d": (C.c_int, [_CTX, C.c_int, C.c_int, _TP, _TP, _I32P, _I32P, _I32P, _I32P]),
     "sg_col2im": (C.c_int, [_CTX, _TP, _TP, _I32P, _I32P, _I32P, _I32P]),
     "sg_softmax_lastaxis": (C.c_int, [_CTX, _TP, _TP, _TP]),
     "sg_softmax_cross_entropy": (C.c_int, [_CTX, _TP, _TP, _TP]),

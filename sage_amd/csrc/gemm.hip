@@ -58,6 +58,16 @@ static __device__ __align__(256) float scratch[SCRATCH_FLOATS];
 constexpr int MAX_DEVICES = 64;
 float *g_scratch_ptr[MAX_DEVICES] = {};  // device address of `scratch` on each GPU, set by sg_gemm_device_setup
 
+// Convolution as a GEMM whose A operand is never materialised: row m of A is output pixel
+// (n, oh, ow), column k is filter tap and channel (ky, kx, c), and A[m][k] is read from the image
+// x[n, oh*sh - ph + ky*dh, ow*sw - pw + kx*dw, c] (zero outside) while the slab is fetched.
+struct ConvG {
+    int H, W, C, OW, KW, ohw;      // image height, width, channels; output width; kernel width; OH*OW
+    int sh, sw, ph, pw, dh, dw;
+    sg_fastdiv d_ohw, d_ow, d_c, d_kw;
+    int vec;                       // C % 4 == 0 and the image is 16-byte aligned: four channels per load
+};
+
 struct GemmP {
     const float *A, *B;
     float *C;
@@ -73,6 +83,7 @@ struct GemmP {
     int vec_c, vec_r, vec_bias;  // 16-byte accesses are legal for C rows / residual rows / the bias
     int k_chunk;      // split-K: workgroup z multiplies k in [z*k_chunk, min(K, (z+1)*k_chunk)); 0 = all of K
     int64_t c_sz;     // split-K: element stride between the partial results of consecutive z
+    ConvG conv;       // used by the CONV instantiations only (A is then the image)
 };
 
 // erf by the five-term rational-exponential form (Abramowitz & Stegun 7.1.26):
@@ -217,8 +228,11 @@ template <int ROWS, bool K_CONTIG> struct Tile {
     }
 };
 
-template <int BM, int BN, int WAVES_M, bool A_KC, bool B_NC, bool GUARD>
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, sg_fastdiv d) { return (__umulhi(n, d.magic) + n) >> d.shift; }
+
+template <int BM, int BN, int WAVES_M, bool A_KC, bool B_NC, bool GUARD, bool CONV = false>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3, 8))) gemm_mfma_kernel(const GemmP p) {
+    static_assert(!CONV || (A_KC && GUARD), "the image-addressed A operand is k-contiguous and goes through the guarded loads");
     constexpr int WAVES_N = 4 / WAVES_M;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -266,7 +280,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     // split-K: this workgroup's share of the k range, addressed from 0 through shifted bases
     const int k_begin = p.k_chunk ? (int)blockIdx.z * p.k_chunk : 0;
     const int Kloc = p.k_chunk ? min(p.K - k_begin, p.k_chunk) : p.K;
-    const float *A = p.A + bt0 * p.a_sb0 + bt1 * p.a_sb1 + (int64_t)k_begin * p.a_sk;
+    const float *A = p.A + bt0 * p.a_sb0 + bt1 * p.a_sb1 + (CONV ? 0 : (int64_t)k_begin * p.a_sk);
     const float *B = p.B + bt0 * p.b_sb0 + bt1 * p.b_sb1 + (int64_t)k_begin * p.b_sk;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -296,12 +310,56 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     for (int i = 0; i < TB::NV; ++i) off_b[i] = TB::lane_offset(i, (uint32_t)p.b_sn, (uint32_t)p.b_sk, tid);
     const __amdgpu_buffer_rsrc_t a_tile = TA::descriptor(TA::tile_base(A, m0, p.a_sm)), b_tile = TB::descriptor(TB::tile_base(B, n0, p.b_sn));
 
+    // CONV: what does not change over the K loop for this thread's items of an A slab: the image of the
+    // item's output pixel, the top-left input coordinates of its window, and its column inside a slab
+    const float *cv_img[TA::NV];
+    int cv_ih0[TA::NV], cv_iw0[TA::NV], cv_k[TA::NV];
+    if (CONV) {
+#pragma unroll
+        for (int i = 0; i < TA::NV; ++i) {
+            int row, k;
+            TA::where(TA::slot(tid + i * NTHREADS), row, k);
+            const uint32_t m = (uint32_t)(m0 + row);
+            const uint32_t n_img = fdiv(m, p.conv.d_ohw), r = m - n_img * (uint32_t)p.conv.ohw;
+            const uint32_t oh = fdiv(r, p.conv.d_ow), ow = r - oh * (uint32_t)p.conv.OW;
+            cv_img[i] = m < (uint32_t)p.M ? p.A + (int64_t)n_img * p.conv.H * p.conv.W * p.conv.C : nullptr;
+            cv_ih0[i] = (int)oh * p.conv.sh - p.conv.ph;
+            cv_iw0[i] = (int)ow * p.conv.sw - p.conv.pw;
+            cv_k[i] = k_begin + k;
+        }
+    }
+    auto conv_load = [&](f32x4 &r, int i, int k0) {
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        const int gk = cv_k[i] + k0, k_lim = k_begin + Kloc;
+        if (cv_img[i] && gk < k_lim) {
+            if (p.conv.vec) {  // four consecutive k are four channels of one tap
+                const uint32_t t = fdiv((uint32_t)gk, p.conv.d_c), c = (uint32_t)gk - t * (uint32_t)p.conv.C;
+                const uint32_t ky = fdiv(t, p.conv.d_kw), kx = t - ky * (uint32_t)p.conv.KW;
+                const int ih = cv_ih0[i] + (int)ky * p.conv.dh, iw = cv_iw0[i] + (int)kx * p.conv.dw;
+                if ((unsigned)ih < (unsigned)p.conv.H && (unsigned)iw < (unsigned)p.conv.W)
+                    v = *reinterpret_cast<const f32x4 *>(cv_img[i] + ((int64_t)ih * p.conv.W + iw) * p.conv.C + c);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (gk + e >= k_lim) break;
+                    const uint32_t t = fdiv((uint32_t)(gk + e), p.conv.d_c), c = (uint32_t)(gk + e) - t * (uint32_t)p.conv.C;
+                    const uint32_t ky = fdiv(t, p.conv.d_kw), kx = t - ky * (uint32_t)p.conv.KW;
+                    const int ih = cv_ih0[i] + (int)ky * p.conv.dh, iw = cv_iw0[i] + (int)kx * p.conv.dw;
+                    if ((unsigned)ih < (unsigned)p.conv.H && (unsigned)iw < (unsigned)p.conv.W)
+                        v[e] = cv_img[i][((int64_t)ih * p.conv.W + iw) * p.conv.C + c];
+                }
+            }
+        }
+        r = v;
+    };
+
     // item e of a slab: global memory -> registers
 #define SG_ITEM_LOAD(e, RA, RB, k0)                                                            \
     do {                                                                                       \
         if ((e) < TA::NV) {                                                                    \
             const int ia = (e) < TA::NV ? (e) : 0;                                         \
-            if (GUARD) TA::load_one_guarded(RA[ia], ia, A, m0, (k0), p.M, Kloc, p.a_sm, p.a_sk, p.vec_a, tid); \
+            if (CONV) conv_load(RA[ia], ia, (k0));                                             \
+            else if (GUARD) TA::load_one_guarded(RA[ia], ia, A, m0, (k0), p.M, Kloc, p.a_sm, p.a_sk, p.vec_a, tid); \
             else TA::load_one_fast(RA[ia], a_tile, off_a[ia], TA::slab_offset((k0), (uint32_t)p.a_sk)); \
         } else {                                                                               \
             const int ib = (e) >= TA::NV ? (e) - TA::NV : 0;                               \
@@ -538,13 +596,23 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *__restr
     float v[W];
 #pragma unroll
     for (int i = 0; i < W; ++i) v[i] = 0.0f;
-    for (int z = 0; z < nsplit; ++z) {
-        if (VEC) {
-            const f32x4 t = *reinterpret_cast<const f32x4 *>(src + z * slice);
+    // eight partial products are requested at a time (one memory round trip per eight) and added in ascending z
+    for (int z0 = 0; z0 < nsplit; z0 += 8) {
+        f32x4 t[8];
 #pragma unroll
-            for (int i = 0; i < W; ++i) v[i] += t[i];
-        } else {
-            v[0] += src[z * slice];
+        for (int u = 0; u < 8; ++u) {
+            t[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (z0 + u < nsplit) {
+                if (VEC) t[u] = *reinterpret_cast<const f32x4 *>(src + (z0 + u) * slice);
+                else t[u].x = src[(z0 + u) * slice];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (z0 + u < nsplit) {
+#pragma unroll
+                for (int i = 0; i < W; ++i) v[i] += t[u][i];
+            }
         }
     }
     const float *R = p.res ? p.res + bt0 * p.r_sb0 + bt1 * p.r_sb1 + (int64_t)m * p.r_sm + n : nullptr;
@@ -569,6 +637,10 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *__restr
 template <int BM, int BN, int WAVES_M, bool GUARD>
 void launch_layouts(sg_ctx *ctx, const GemmP &p, dim3 grid, bool a_kc, bool b_nc) {
     dim3 block(NTHREADS);
+    if (p.conv.ohw) {  // image-addressed A (sg_conv2d): one instantiation per tile shape
+        if constexpr (GUARD) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, true, true>), grid, block, 0, ctx->stream, p);
+        return;
+    }
     if (a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD>), grid, block, 0, ctx->stream, p);
     else if (a_kc && !b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, false, GUARD>), grid, block, 0, ctx->stream, p);
     else if (!a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, true, GUARD>), grid, block, 0, ctx->stream, p);
@@ -583,20 +655,25 @@ bool needs_guard(const GemmP &p, int bm, int bn, bool a_kc, bool b_nc) {
     const int64_t reach_b = b_nc ? (int64_t)p.K * p.b_sk + bn : (int64_t)bn * p.b_sn + p.K;
     const bool fits32 = reach_a >= 0 && reach_b >= 0 && reach_a < (1ll << 29) && reach_b < (1ll << 29);
     const bool vec_out = p.vec_c && (!p.res || p.vec_r) && (!p.bias || p.vec_bias);
+    if (p.conv.ohw) return true;
     return p.M % bm != 0 || p.N % bn != 0 || p.K % (2 * BK) != 0 || !p.vec_a || !p.vec_b || !vec_out || !fits32;
 }
 
 // How many k ranges to split into.  Splitting pays when the output has too few tiles to occupy the
 // chip and K is long: each range becomes its own workgroup (grid z) writing a partial product, and a
 // second kernel sums them.  Ranges are multiples of 32 so that the unguarded loop stays legal.
-int choose_split(int num_cus, int64_t wgs, int K, int *k_chunk) {
+int choose_split(int num_cus, int64_t wgs, int K, bool image_operand, int *k_chunk) {
     const int64_t cus = num_cus > 0 ? num_cus : 256;
     *k_chunk = 0;
     const char *force = getenv("SAGE_GEMM_SPLITK");
     int want;
     if (force) want = atoi(force);
     else {
-        if (wgs * 2 > cus || K < 512) return 1;
+        // One 64x64 tile per compute unit multiplies 16 of k in about 0.21 us; the second pass and the extra launch
+        // cost about 11 us more than they save below K = 1024 (measured at 64..98 workgroups, K = 512..1152).
+        // With the A operand read from an image every slab also pays the window arithmetic, and splitting
+        // pays from K = 512 (ResNet-18 forward: 0.365 against 0.398 ms).
+        if (wgs * 2 > cus || K < (image_operand ? 512 : 1024)) return 1;
         want = (int)((2 * cus + wgs - 1) / wgs);
         if (want > K / 128) want = K / 128;
         if (want > 32) want = 32;
@@ -609,51 +686,54 @@ int choose_split(int num_cus, int64_t wgs, int K, int *k_chunk) {
     return nsplit;
 }
 
+// Where the partial products of a split-K product go: a block from the context's allocator (it counts against
+// the capacity; when it does not fit the call fails with SG_ERR_OOM like any other allocation, and the caller's
+// eviction loop, session.rs:259-325, frees memory and calls again, instead of silently taking a single-pass
+// kernel whose rounding differs), or the static per-device array for the entry point that allocates nothing.
+int workspace(sg_ctx *ctx, int64_t floats, bool noalloc, void **ws) {
+    if (!noalloc) return sg_alloc(ctx, (uint64_t)floats * sizeof(float), ws);
+    if (floats > SCRATCH_FLOATS)
+        return sg_fail(ctx, SG_ERR_ARG, "sg_gemm_noalloc: this product runs split-K and needs %lld bytes of workspace, "
+                       "more than the %lld-byte static scratch (use sg_gemm)", (long long)floats * 4, (long long)SCRATCH_FLOATS * 4);
+    *ws = ctx->device >= 0 && ctx->device < MAX_DEVICES ? g_scratch_ptr[ctx->device] : nullptr;
+    if (!*ws) return sg_fail(ctx, SG_ERR_DEVICE, "sg_gemm_noalloc: the static scratch of device %d was not set up", ctx->device);
+    return SG_OK;
+}
+
+// The first pass of a split-K product: raw partial products [split][batch][M][N] into the workspace, no epilogue.
+GemmP partial_pass(const GemmP &p, float *ws, int64_t slice, int k_chunk) {
+    GemmP q = p;
+    q.C = ws;
+    q.c_sm = p.N; q.c_sb1 = (int64_t)p.M * p.N; q.c_sb0 = q.c_sb1 * p.nb1; q.c_sz = slice;
+    q.k_chunk = k_chunk;
+    q.bias = nullptr; q.res = nullptr; q.alpha = 1.0f; q.act = SG_ACT_NONE; q.act_post = SG_ACT_NONE;
+    q.vec_c = p.N % 4 == 0;
+    return q;
+}
+
+void launch_splitk_reduce(sg_ctx *ctx, const GemmP &p, const float *ws, int nsplit, int64_t slice);
+
 template <int BM, int BN, int WAVES_M>
 int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noalloc) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     int k_chunk = 0;
-    const int nsplit = choose_split(ctx->num_cus, (int64_t)p.tiles_m * p.tiles_n * batch, p.K, &k_chunk);
+    const int nsplit = choose_split(ctx->num_cus, (int64_t)p.tiles_m * p.tiles_n * batch, p.K, p.conv.ohw != 0, &k_chunk);
     if (nsplit > 1) {
         const int64_t slice = (int64_t)batch * p.M * p.N;
-        // The workspace comes from the context's allocator and counts against its capacity.  When it
-        // does not fit the call fails with SG_ERR_OOM like any other allocation (the caller's
-        // eviction loop, session.rs:259-325, frees memory and calls again) instead of silently taking
-        // the single-pass kernel, whose rounding differs: the same call always gives the same bits.
         void *ws = nullptr;
-        if (noalloc) {
-            // the per-device static array instead: nothing is allocated, larger products are refused
-            if ((int64_t)nsplit * slice > SCRATCH_FLOATS)
-                return sg_fail(ctx, SG_ERR_ARG, "sg_gemm_noalloc: this product runs split-K over %d ranges and needs %lld bytes of workspace, "
-                               "more than the %lld-byte static scratch (use sg_gemm)", nsplit, (long long)nsplit * slice * 4, (long long)SCRATCH_FLOATS * 4);
-            ws = ctx->device >= 0 && ctx->device < MAX_DEVICES ? g_scratch_ptr[ctx->device] : nullptr;
-            if (!ws) return sg_fail(ctx, SG_ERR_DEVICE, "sg_gemm_noalloc: the static scratch of device %d was not set up", ctx->device);
-        } else {
-            const int rc_ws = sg_alloc(ctx, (uint64_t)nsplit * slice * sizeof(float), &ws);
-            if (rc_ws != SG_OK) return rc_ws;
-        }
-        {
-            GemmP q = p;  // first pass: raw partial products into the workspace
-            q.C = (float *)ws;
-            q.c_sm = p.N; q.c_sb1 = (int64_t)p.M * p.N; q.c_sb0 = q.c_sb1 * p.nb1; q.c_sz = slice;
-            q.k_chunk = k_chunk;
-            q.bias = nullptr; q.res = nullptr; q.alpha = 1.0f; q.act = SG_ACT_NONE; q.act_post = SG_ACT_NONE;
-            q.vec_c = p.N % 4 == 0;
-            dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, (unsigned)nsplit);
-            if (needs_guard(q, BM, BN, a_kc, b_nc)) launch_layouts<BM, BN, WAVES_M, true>(ctx, q, grid, a_kc, b_nc);
-            else launch_layouts<BM, BN, WAVES_M, false>(ctx, q, grid, a_kc, b_nc);
-            SG_CHECK_LAUNCH(ctx, "gemm (split-K pass 1)");
-            const bool vec = p.N % 4 == 0;
-            const int64_t total = slice / (vec ? 4 : 1);
-            dim3 rgrid((unsigned)((total + 255) / 256));
-            if (vec) hipLaunchKernelGGL((splitk_reduce_kernel<true>), rgrid, dim3(256), 0, ctx->stream, (const float *)ws, nsplit, slice, p, total);
-            else hipLaunchKernelGGL((splitk_reduce_kernel<false>), rgrid, dim3(256), 0, ctx->stream, (const float *)ws, nsplit, slice, p, total);
-            SG_CHECK_LAUNCH(ctx, "gemm (split-K pass 2)");
-            if (noalloc) return SG_OK;  // the static scratch stays; the next call on this stream is ordered behind pass 2
-            // the block returns to the context's cache; later users are ordered behind these kernels on the stream
-            return sg_free(ctx, ws);
-        }
+        const int rc_ws = workspace(ctx, (int64_t)nsplit * slice, noalloc, &ws);
+        if (rc_ws != SG_OK) return rc_ws;
+        GemmP q = partial_pass(p, (float *)ws, slice, k_chunk);
+        dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, (unsigned)nsplit);
+        if (needs_guard(q, BM, BN, a_kc, b_nc)) launch_layouts<BM, BN, WAVES_M, true>(ctx, q, grid, a_kc, b_nc);
+        else launch_layouts<BM, BN, WAVES_M, false>(ctx, q, grid, a_kc, b_nc);
+        SG_CHECK_LAUNCH(ctx, "gemm (split-K pass 1)");
+        launch_splitk_reduce(ctx, p, (const float *)ws, nsplit, slice);
+        SG_CHECK_LAUNCH(ctx, "gemm (split-K pass 2)");
+        // the static scratch stays; a block from the allocator returns to the context's cache (later users of either
+        // are ordered behind these kernels on the stream)
+        return noalloc ? SG_OK : sg_free(ctx, ws);
     }
     // one workgroup per tile while they all fit at once (three per compute unit), else that many workgroups
     // walking the tiles; a batched product keeps one workgroup per tile and batch entry
@@ -692,6 +772,14 @@ int choose_tile(int num_cus, int M, int N, int batch) {
     return best;
 }
 
+void launch_splitk_reduce(sg_ctx *ctx, const GemmP &p, const float *ws, int nsplit, int64_t slice) {
+    const bool vec = p.N % 4 == 0;
+    const int64_t total = slice / (vec ? 4 : 1);
+    dim3 rgrid((unsigned)((total + 255) / 256));
+    if (vec) hipLaunchKernelGGL((splitk_reduce_kernel<true>), rgrid, dim3(256), 0, ctx->stream, ws, nsplit, slice, p, total);
+    else hipLaunchKernelGGL((splitk_reduce_kernel<false>), rgrid, dim3(256), 0, ctx->stream, ws, nsplit, slice, p, total);
+}
+
 int launch_gemm(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noalloc) {
     switch (choose_tile(ctx->num_cus, p.M, p.N, batch)) {
     case 0: return launch_cfg<128, 128, 2>(ctx, p, batch, a_kc, b_nc, noalloc);
@@ -709,7 +797,8 @@ struct Mat {
     int64_t sb0, sb1, s_row, s_col;
 };
 
-int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c, const sg_gemm_epilogue *epi, bool noalloc = false) {
+int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c, const sg_gemm_epilogue *epi, bool noalloc = false,
+        const ConvG *conv = nullptr) {
     if (M < 1 || N < 1 || K < 1) return sg_fail(ctx, SG_ERR_SHAPE, "gemm: empty dimension");
     // Which axis of each operand is the contiguous one.  An axis of extent 1 may carry any stride.
     bool a_kc, b_nc;
@@ -730,6 +819,7 @@ int run(sg_ctx *ctx, int M, int N, int K, int nb0, int nb1, Mat a, Mat b, Mat c,
     p.a_sm = a.s_row; p.a_sk = a.s_col; p.b_sk = b.s_row; p.b_sn = b.s_col; p.c_sm = c.s_row;
     p.a_sb0 = a.sb0; p.a_sb1 = a.sb1; p.b_sb0 = b.sb0; p.b_sb1 = b.sb1; p.c_sb0 = c.sb0; p.c_sb1 = c.sb1;
     p.nb1 = nb1;
+    if (conv) p.conv = *conv;
     p.alpha = 1.0f; p.act = SG_ACT_NONE; p.act_post = SG_ACT_NONE;
     auto mult4 = [](int64_t v) { return v % 4 == 0; };
     p.vec_a = ptr_aligned16(a.ptr) && mult4(a_kc ? p.a_sm : p.a_sk) && mult4(a.sb0) && mult4(a.sb1);
@@ -828,6 +918,43 @@ extern "C" int sg_gemm(sg_ctx *ctx, int ta, int tb, const sg_tensor *a, const sg
 extern "C" int sg_gemm_noalloc(sg_ctx *ctx, int ta, int tb, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c,
                                const sg_gemm_epilogue *epi) {
     return gemm_rank2(ctx, ta, tb, a, b, c, epi, true);
+}
+
+// conv_2d (conv.rs:61-96) in one launch: the [N*OH*OW, KH*KW*C] column matrix of im2col is never written;
+// the GEMM's A operand is read from the image through the window arithmetic of Im2col (conv.rs:304-349).
+extern "C" int sg_conv2d(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *filter, const sg_tensor *out, const int32_t stride[2],
+                         const int32_t pad[2], const int32_t dil[2], const sg_gemm_epilogue *epi) {
+    if (!ctx || !stride || !pad || !dil) return SG_ERR_ARG;
+    int rc = check_f32(ctx, x, filter, out, "sg_conv2d");
+    if (rc != SG_OK) return rc;
+    if (x->rank != 4 || filter->rank != 4 || out->rank != 4) return sg_fail(ctx, SG_ERR_SHAPE, "sg_conv2d: x [N,H,W,C], filter [KH,KW,C,OC], out [N,OH,OW,OC] (conv.rs:70, 199)");
+    if (!sg_is_dense(x) || !sg_is_dense(filter) || !sg_is_dense(out)) return sg_fail(ctx, SG_ERR_SHAPE, "sg_conv2d: operands must be dense (conv.rs:200)");
+    for (int i = 0; i < 2; ++i)
+        if (stride[i] < 1 || pad[i] < 0 || dil[i] < 0) return sg_fail(ctx, SG_ERR_ARG, "sg_conv2d: bad geometry");
+    const int64_t N = x->extents[0], H = x->extents[1], W = x->extents[2], Cc = x->extents[3];
+    const int64_t KH = filter->extents[0], KW = filter->extents[1], OC = filter->extents[3];
+    if (filter->extents[2] != Cc) return sg_fail(ctx, SG_ERR_SHAPE, "sg_conv2d: filter has %lld input channels, the image %lld (conv.rs:86)", (long long)filter->extents[2], (long long)Cc);
+    // conv_size (conv.rs:47-59); every pair is {w, h}
+    const int64_t OW = (W + 2 * pad[0] - (int64_t)dil[0] * (KW - 1) - 1) / stride[0] + 1;
+    const int64_t OH = (H + 2 * pad[1] - (int64_t)dil[1] * (KH - 1) - 1) / stride[1] + 1;
+    if (OW < 1 || OH < 1) return sg_fail(ctx, SG_ERR_SHAPE, "sg_conv2d: kernel larger than padded image");
+    const int64_t want[4] = {N, OH, OW, OC};
+    for (int a = 0; a < 4; ++a)
+        if (out->extents[a] != want[a]) return sg_fail(ctx, SG_ERR_SHAPE, "sg_conv2d: out extent[%d] = %lld, expected %lld", a, (long long)out->extents[a], (long long)want[a]);
+    const int64_t M = N * OH * OW, K = KH * KW * Cc;
+    if (M >= (1ll << 31) || K >= (1ll << 31)) return sg_fail(ctx, SG_ERR_SHAPE, "sg_conv2d: more than 2^31-1 output pixels or filter taps");
+    ConvG g{};
+    g.H = (int)H; g.W = (int)W; g.C = (int)Cc; g.OW = (int)OW; g.KW = (int)KW; g.ohw = (int)(OH * OW);
+    g.sw = stride[0]; g.sh = stride[1]; g.pw = pad[0]; g.ph = pad[1]; g.dw = dil[0]; g.dh = dil[1];
+    g.d_ohw = sg_make_fastdiv((uint32_t)g.ohw); g.d_ow = sg_make_fastdiv((uint32_t)OW);
+    g.d_c = sg_make_fastdiv((uint32_t)Cc); g.d_kw = sg_make_fastdiv((uint32_t)KW);
+    const float *img = (const float *)x->base + x->offset;
+    g.vec = Cc % 4 == 0 && ptr_aligned16(img);
+    // A = the virtual [M, K] column matrix (row stride K, never dereferenced through it), B = filter as [K, OC], C = out as [M, OC]
+    Mat ma{img, 0, 0, K, 1};
+    Mat mb{(const float *)filter->base + filter->offset, 0, 0, OC, 1};
+    Mat mc{(const float *)out->base + out->offset, 0, 0, OC, 1};
+    return run(ctx, (int)M, (int)OC, (int)K, 1, 1, ma, mb, mc, epi, false, &g);
 }
 
 // Called by sg_ctx_create with the context's device current: resolves the device address of `scratch`

@@ -89,6 +89,55 @@ struct Im2colP {
     int batch, chan, img_w, img_h, col_w, col_h, ker_w, ker_h, stride_w, stride_h, pad_w, pad_h, dil_w, dil_h;
 };
 
+// Pooling without the column tensor: out[n, oy, ox, c] = reduce over (ky, kx) of the window the reference's
+// max_pool_2d / avg_pool_2d first copy out with im2col and then reduce over axes [3, 4] (conv.rs:143-165).
+// Pixels outside the image count as zeros, as they do in the column tensor; the accumulator starts at 0
+// (ref_zero, reduce.rs:282) or at the operator's identity; the window is walked in the order of the
+// reference's reduce kernel (first reduced axis, ky, innermost).  One thread per VEC channels of one output pixel.
+template <int VEC>
+__global__ void __launch_bounds__(256) pool2d_kernel(const float *__restrict__ img, float *__restrict__ out, uint32_t n_vec, Im2colP p,
+                                                     int op, int ref_zero) {
+    uint32_t gid = blockIdx.x * 256u + threadIdx.x;
+    if (gid >= n_vec) return;
+    const uint32_t cv = p.chan / VEC;
+    uint32_t rem = gid;
+    const uint32_t c = (rem % cv) * VEC; rem /= cv;
+    const uint32_t ox = rem % p.col_w; rem /= p.col_w;
+    const uint32_t oy = rem % p.col_h; rem /= p.col_h;
+    const uint32_t n = rem;
+    const float start = ref_zero ? 0.0f : (op == SG_R_SUM ? 0.0f : op == SG_R_PROD ? 1.0f : op == SG_R_MAX ? -__builtin_inff() : __builtin_inff());
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = start;
+    const float *base = img + (size_t)n * p.img_h * p.img_w * p.chan + c;
+    for (int kx = 0; kx < p.ker_w; ++kx) {
+        const int ix = (int)ox * p.stride_w - p.pad_w + kx * p.dil_w;
+        for (int ky = 0; ky < p.ker_h; ++ky) {
+            const int iy = (int)oy * p.stride_h - p.pad_h + ky * p.dil_h;
+            float v[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[e] = 0.0f;
+            if (ix >= 0 && ix < p.img_w && iy >= 0 && iy < p.img_h) {
+                const float *q = base + ((size_t)iy * p.img_w + ix) * p.chan;
+                if (VEC == 4) {
+                    const float4 t = *reinterpret_cast<const float4 *>(q);
+                    v[0] = t.x; v[1 % VEC] = t.y; v[2 % VEC] = t.z; v[3 % VEC] = t.w;
+                } else {
+                    v[0] = q[0];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float a = acc[e], b = v[e];
+                acc[e] = op == SG_R_SUM ? a + b : op == SG_R_PROD ? a * b : op == SG_R_MAX ? (a < b ? b : a) : (b < a ? b : a);
+            }
+        }
+    }
+    float *dst = out + (size_t)gid * VEC;
+    if (VEC == 4) *reinterpret_cast<float4 *>(dst) = make_float4(acc[0], acc[1 % VEC], acc[2 % VEC], acc[3 % VEC]);
+    else dst[0] = acc[0];
+}
+
 // One thread per VEC consecutive channels of one (n, oy, ox, ky, kx) cell of the column tensor.
 template <int VEC>
 __global__ void __launch_bounds__(256) im2col_kernel(const float *__restrict__ img, float *__restrict__ col, uint32_t n_vec, Im2colP p) {
@@ -304,6 +353,47 @@ extern "C" int sg_im2col(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, 
         hipLaunchKernelGGL((im2col_kernel<1>), dim3((n + 255) / 256), dim3(256), 0, ctx->stream, img, col, n, p);
     }
     SG_CHECK_LAUNCH(ctx, "im2col");
+    return SG_OK;
+}
+
+extern "C" int sg_pool2d(sg_ctx *ctx, int op, int init_mode, const sg_tensor *x, const sg_tensor *out, const int32_t ker[2],
+                         const int32_t stride[2], const int32_t pad[2], const int32_t dil[2]) {
+    if (!ctx || !ker || !stride || !pad || !dil) return SG_ERR_ARG;
+    int rc;
+    if ((rc = sg_validate_tensor(ctx, x, "sg_pool2d x")) != SG_OK) return rc;
+    if ((rc = sg_validate_tensor(ctx, out, "sg_pool2d out")) != SG_OK) return rc;
+    if (op < SG_R_SUM || op > SG_R_MIN) return sg_fail(ctx, SG_ERR_ARG, "sg_pool2d: unknown op %d", op);
+    if (init_mode != SG_INIT_REF_ZERO && init_mode != SG_INIT_IDENTITY) return sg_fail(ctx, SG_ERR_ARG, "sg_pool2d: bad init_mode");
+    if (x->dtype != SG_FLOAT || out->dtype != SG_FLOAT) return sg_fail(ctx, SG_ERR_DTYPE, "sg_pool2d: fp32 only (conv.rs:337 reads float)");
+    if (x->rank != 4 || out->rank != 4) return sg_fail(ctx, SG_ERR_SHAPE, "sg_pool2d: x must be [N,H,W,C], out [N,OH,OW,C] (conv.rs:199)");
+    if (!sg_is_dense(x) || !sg_is_dense(out)) return sg_fail(ctx, SG_ERR_SHAPE, "sg_pool2d: x and out must be dense (conv.rs:200)");
+    for (int i = 0; i < 2; ++i)
+        if (ker[i] < 1 || stride[i] < 1 || pad[i] < 0 || dil[i] < 0) return sg_fail(ctx, SG_ERR_ARG, "sg_pool2d: bad geometry");
+    Im2colP p;
+    p.batch = (int)x->extents[0]; p.img_h = (int)x->extents[1]; p.img_w = (int)x->extents[2]; p.chan = (int)x->extents[3];
+    p.ker_w = ker[0]; p.ker_h = ker[1]; p.stride_w = stride[0]; p.stride_h = stride[1];
+    p.pad_w = pad[0]; p.pad_h = pad[1]; p.dil_w = dil[0]; p.dil_h = dil[1];
+    // conv_size (conv.rs:47-59)
+    const int64_t ow = ((int64_t)p.img_w + 2 * p.pad_w - (int64_t)p.dil_w * (p.ker_w - 1) - 1) / p.stride_w + 1;
+    const int64_t oh = ((int64_t)p.img_h + 2 * p.pad_h - (int64_t)p.dil_h * (p.ker_h - 1) - 1) / p.stride_h + 1;
+    if (ow < 1 || oh < 1) return sg_fail(ctx, SG_ERR_SHAPE, "sg_pool2d: kernel larger than padded image");
+    p.col_w = (int)ow; p.col_h = (int)oh;
+    const int64_t want[4] = {p.batch, oh, ow, p.chan};
+    for (int a = 0; a < 4; ++a)
+        if (out->extents[a] != want[a]) return sg_fail(ctx, SG_ERR_SHAPE, "sg_pool2d: out extent[%d] = %lld, expected %lld", a, (long long)out->extents[a], (long long)want[a]);
+    const float *img = (const float *)x->base + x->offset;
+    float *dst = (float *)out->base + out->offset;
+    const int64_t total = sg_numel(out);
+    const int ref_zero = init_mode == SG_INIT_REF_ZERO;
+    const bool vec = p.chan % 4 == 0 && ((uintptr_t)img % 16 == 0) && ((uintptr_t)dst % 16 == 0);
+    if (vec) {
+        const uint32_t n = (uint32_t)(total / 4);
+        hipLaunchKernelGGL((pool2d_kernel<4>), dim3((n + 255) / 256), dim3(256), 0, ctx->stream, img, dst, n, p, op, ref_zero);
+    } else {
+        const uint32_t n = (uint32_t)total;
+        hipLaunchKernelGGL((pool2d_kernel<1>), dim3((n + 255) / 256), dim3(256), 0, ctx->stream, img, dst, n, p, op, ref_zero);
+    }
+    SG_CHECK_LAUNCH(ctx, "pool2d");
     return SG_OK;
 }
 

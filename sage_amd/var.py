@@ -1053,6 +1053,22 @@ class _Evaluator:
 
     # ---- reductions and indexing
     def _ev_reduce(self, v):
+        col = v.inputs[0]
+        if (_FUSION["on"] and col.op == "im2col" and self._private(col) and sorted(v.attrs["axes"]) == [3, 4]
+                and v.dtype == FLOAT and os.environ.get("SAGE_FUSE_CONV", "1") != "0"):
+            # max_pool_2d / avg_pool_2d (conv.rs:143-165): the window is reduced while it is read, no column tensor
+            x = self.get(col.inputs[0])
+            if not x.is_dense():
+                x = self.run_copy(x)
+            n, oh, ow, _, _, c = col.extents
+            y = self.out(v.extents, FLOAT)
+            a = col.attrs
+            arr = lambda p: (C.c_int32 * 2)(*p)
+            op = {"sum": abi.R_SUM, "prod": abi.R_PROD, "max": abi.R_MAX, "min": abi.R_MIN}[v.attrs["op"]]
+            init = abi.INIT_REF_ZERO if v.attrs["init"] == "ref_zero" else abi.INIT_IDENTITY
+            xc, yc = x.c(), y.with_shape(Shape([n, oh, ow, c])).c()
+            self.call(self.lib.sg_pool2d, op, init, C.byref(xc), C.byref(yc), arr(a["ker"]), arr(a["stride"]), arr(a["pad"]), arr(a["dil"]))
+            return y
         x = self.get(v.inputs[0])
         y = self.out(v.extents, v.dtype)
         axes = v.attrs["axes"]
@@ -1159,6 +1175,10 @@ class _Evaluator:
     def run_gemm(self, g, epi=None, dest=None):
         """Run gemm / gemm_batched / matmul_nd node `g`.  `dest`: a Tensor view with g's extents to
         write into (any batch strides, unit last stride); default a fresh dense tensor."""
+        if _FUSION["on"] and dest is None:
+            t = self.try_conv(g, epi)
+            if t is not None:
+                return t
         a, b = self.get(g.inputs[0]), self.get(g.inputs[1])
         keep = self.keepalive
         e = self._epi_struct(epi, keep)
@@ -1184,6 +1204,40 @@ class _Evaluator:
         ac, bc, yc = a.c(), b.c(), y.c()
         fn = self.lib.sg_gemm if g.op == "gemm" else self.lib.sg_gemm_batched
         self.call(fn, int(g.attrs["ta"]), int(g.attrs["tb"]), C.byref(ac), C.byref(bc), C.byref(yc), ep)
+        return y
+
+    def try_conv(self, g, epi):
+        """conv_2d's `view(im2col(x)) . view(filter)` (conv.rs:61-96) as one sg_conv2d launch: the column
+        matrix is consumed by this product only, so it is never written."""
+        if g.op != "gemm" or g.attrs["ta"] or g.attrs["tb"] or os.environ.get("SAGE_FUSE_CONV", "1") == "0":
+            return None
+        col = g.inputs[0]
+        while col.op == "reshape" and self._private(col):
+            col = col.inputs[0]
+        if col.op != "im2col" or not self._private(col):
+            return None
+        f = g.inputs[1]
+        while f.op == "reshape" and f.value is None:
+            f = f.inputs[0]
+        a = col.attrs
+        n, oh, ow, kh, kw, c = col.extents
+        if f.rank != 4 or f.extents[:3] != [kh, kw, c] or a["ker"] != [kw, kh]:
+            return None
+        x, ft = self.get(col.inputs[0]), self.get(f)
+        if not x.is_dense():
+            x = self.run_copy(x)
+        if not ft.is_dense():
+            ft = self.run_copy(ft)
+        keep = self.keepalive
+        e = self._epi_struct(epi, keep)
+        if e is not None:
+            keep.append(e)
+        y = self.out(g.extents, FLOAT)
+        arr = lambda p: (C.c_int32 * 2)(*p)
+        xc, fc = x.c(), ft.c()
+        yc = y.with_shape(Shape([n, oh, ow, g.extents[1]])).c()
+        self.call(self.lib.sg_conv2d, C.byref(xc), C.byref(fc), C.byref(yc), arr(a["stride"]), arr(a["pad"]), arr(a["dil"]),
+                  C.byref(e) if e is not None else None)
         return y
 
     def _ev_gemm(self, v):

@@ -592,6 +592,100 @@ def test_conv_and_pools(ctx):
     close(V.avg_pool_2d(dev(ctx, xp), 2, 2, 0, 1).eval(ctx).numpy(), O.avg_pool_2d(ht(xp), 2, 2, 0, 1).numpy(), REL_MAP, "avg_pool")
 
 
+CONV_CASES = [
+    # (n, h, w, c, kh, kw, oc, stride [w,h], pad [w,h], dil [w,h])
+    (2, 12, 10, 5, 3, 3, 7, [2, 2], [1, 1], [1, 1]),      # channels not a multiple of 4: scalar taps
+    (3, 28, 28, 1, 7, 7, 64, [2, 2], [3, 3], [1, 1]),     # the first ResNet convolution: one channel, K = 49
+    (4, 14, 14, 64, 3, 3, 64, [1, 1], [1, 1], [1, 1]),    # 16-byte channel loads, exactly tiled N
+    (2, 9, 11, 8, 3, 2, 12, [1, 2], [2, 0], [2, 1]),      # rectangular kernel, mixed stride/padding, dilation
+    (2, 7, 7, 128, 1, 1, 256, [2, 2], [0, 0], [1, 1]),    # 1x1 stride-2 downsample
+    (16, 4, 4, 256, 3, 3, 256, [1, 1], [1, 1], [1, 1]),   # few output tiles and K = 2304: split-K
+    (1, 6, 6, 4, 3, 3, 8, [1, 1], [1, 1], [0, 0]),        # dilation 0 (every tap reads the window's corner, as the reference would)
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=[f"c{i}" for i in range(len(CONV_CASES))])
+def test_conv2d_without_column_matrix(ctx, monkeypatch, case):
+    """sg_conv2d reads the GEMM's A operand from the image through the im2col window arithmetic.  It must
+    equal the oracle's im2col + gemm (conv.rs:61-96) within the GEMM tolerance, and the explicit
+    sg_im2col + sg_gemm path bit for bit where both split K the same way (same tiles, same k order; between
+    K = 512 and 1024 only the image-addressed product is split), with and without bias / ReLU / residual."""
+    n, h, w, c, kh, kw, oc, stride, pad, dil = case
+    say("conv2d", case)
+    rng = np.random.default_rng(n * 100 + c)
+    x = rng.standard_normal((n, h, w, c)).astype(np.float32)
+    f = (rng.standard_normal((kh, kw, c, oc)) * 0.2).astype(np.float32)
+    bias = rng.standard_normal((oc,)).astype(np.float32)
+
+    def build(with_epilogue):
+        y = V.conv_2d(dev(ctx, x), dev(ctx, f), stride, pad, dil)
+        if with_epilogue:
+            y = nn.relu(y + dev(ctx, bias)) + dev(ctx, res)
+        return y
+
+    yo = O.conv_2d(ht(x), ht(f), stride, pad, dil)
+    res = rng.standard_normal(tuple(yo.extents)).astype(np.float32)
+    for with_epilogue in (False, True):
+        n0 = ctx.launches
+        y_fused = build(with_epilogue).eval(ctx).numpy()
+        fused_launches = ctx.launches - n0
+        monkeypatch.setenv("SAGE_FUSE_CONV", "0")
+        y_explicit = build(with_epilogue).eval(ctx).numpy()
+        monkeypatch.delenv("SAGE_FUSE_CONV")
+        ref = yo.numpy()
+        if with_epilogue:
+            ref = O.binary("add", O.relu(O.binary("add", yo, ht(bias))), ht(res)).numpy()
+        close(y_fused, ref, REL_GEMM, "conv2d vs oracle")
+        if 512 <= kh * kw * c < 1024:
+            close(y_fused, y_explicit, REL_GEMM, "conv2d vs im2col + gemm")
+        else:
+            exact(y_fused, y_explicit, "conv2d vs im2col + gemm")
+        assert fused_launches <= (2 if with_epilogue else 1), fused_launches
+
+
+@pytest.mark.parametrize("geom", [((2, 12, 10, 8), 3, 2, 1, 1), ((3, 14, 14, 64), 3, 2, 1, 1), ((2, 9, 7, 5), [2, 3], [1, 2], [1, 0], [2, 1]),
+                                  ((4, 7, 7, 16), 7, 7, 0, 1), ((1, 6, 6, 3), 2, 2, 0, 1)])
+def test_pooling_without_column_tensor(ctx, monkeypatch, geom):
+    """max_pool_2d / avg_pool_2d (conv.rs:143-165) as one window kernel: bit-exact against the oracle's
+    im2col + reduce for max (negative inputs included: the reference's accumulator starts at 0 and padding
+    pixels are zeros), within the reduction tolerance for the mean, and equal to the two-launch path."""
+    shape, ker, stride, pad, dil = geom
+    say("pool2d", geom)
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal(shape).astype(np.float32)
+    n0 = ctx.launches
+    ymax = V.max_pool_2d(dev(ctx, x), ker, stride, pad, dil).eval(ctx).numpy()
+    assert ctx.launches - n0 == 1
+    exact(ymax, O.max_pool_2d(ht(x), ker, stride, pad, dil).numpy(), "max_pool vs oracle")
+    yavg = V.avg_pool_2d(dev(ctx, x), ker, stride, pad, dil).eval(ctx).numpy()
+    close(yavg, O.avg_pool_2d(ht(x), ker, stride, pad, dil).numpy(), REL_MAP, "avg_pool vs oracle")
+    ymin = V.im2col(dev(ctx, x), ker, stride, pad, dil).min([3, 4], True).eval(ctx).numpy()
+    monkeypatch.setenv("SAGE_FUSE_CONV", "0")
+    exact(ymax, V.max_pool_2d(dev(ctx, x), ker, stride, pad, dil).eval(ctx).numpy(), "max_pool vs im2col + reduce")
+    close(yavg, V.avg_pool_2d(dev(ctx, x), ker, stride, pad, dil).eval(ctx).numpy(), REL_MAP, "avg_pool vs im2col + reduce")
+    exact(ymin, V.im2col(dev(ctx, x), ker, stride, pad, dil).min([3, 4], True).eval(ctx).numpy(), "min with preserved axes")
+
+
+def test_conv2d_abi_errors(ctx):
+    say("conv2d error behaviour")
+    lib = abi.lib()
+    x = S.Tensor.from_numpy(ctx, np.zeros((1, 5, 5, 4), np.float32))
+    f = S.Tensor.from_numpy(ctx, np.zeros((3, 3, 4, 8), np.float32))
+    f_bad = S.Tensor.from_numpy(ctx, np.zeros((3, 3, 5, 8), np.float32))
+    out = S.Tensor.uninit(ctx, [1, 5, 5, 8])
+    out_bad = S.Tensor.uninit(ctx, [1, 4, 5, 8])
+    arr = lambda a, b: (C.c_int32 * 2)(a, b)
+    xc, fc, fbc, oc, obc = x.c(), f.c(), f_bad.c(), out.c(), out_bad.c()
+    assert lib.sg_conv2d(ctx.handle, C.byref(xc), C.byref(fc), C.byref(oc), arr(1, 1), arr(1, 1), arr(1, 1), None) == abi.OK
+    assert lib.sg_conv2d(ctx.handle, C.byref(xc), C.byref(fbc), C.byref(oc), arr(1, 1), arr(1, 1), arr(1, 1), None) == abi.ERR_SHAPE  # conv.rs:86
+    assert lib.sg_conv2d(ctx.handle, C.byref(xc), C.byref(fc), C.byref(obc), arr(1, 1), arr(1, 1), arr(1, 1), None) == abi.ERR_SHAPE
+    assert lib.sg_conv2d(ctx.handle, C.byref(xc), C.byref(fc), C.byref(oc), arr(0, 1), arr(1, 1), arr(1, 1), None) == abi.ERR_ARG
+    big = S.Tensor.from_numpy(ctx, np.zeros((9, 9, 4, 8), np.float32))
+    bc = big.c()
+    assert lib.sg_conv2d(ctx.handle, C.byref(xc), C.byref(bc), C.byref(oc), arr(1, 1), arr(0, 0), arr(1, 1), None) == abi.ERR_SHAPE  # kernel larger than image
+    ctx.sync()
+
+
 # ----------------------------------------------------------------------------- fused row operators
 @pytest.mark.parametrize("shape", [(64, 128), (5, 1000), (3, 4, 16, 16), (9, 1024), (2, 2052), (7, 10)])
 def test_softmax_fused_vs_composed_vs_oracle(ctx, shape):

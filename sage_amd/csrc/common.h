@@ -22,6 +22,12 @@ struct sg_jit_kernel {
     hipFunction_t fn;
 };
 
+// What a repeat call of the same map operator needs: the built kernel and the dtype its expression yields.
+struct sg_map_entry {
+    hipFunction_t fn;
+    int result_dtype;
+};
+
 // Context (session/context.rs:25-36): device + stream + kernel cache + allocator.
 struct sg_ctx {
     int device = 0;
@@ -36,6 +42,10 @@ struct sg_ctx {
     std::multimap<uint64_t, void *> cache;
     // run-time built kernels keyed by their full source text (session/context.rs:62-83)
     std::unordered_map<std::string, sg_jit_kernel> jit;
+    // the same kernels by operator signature (expression program, operand dtypes and layout classes): a repeat
+    // call of an operator finds its kernel without generating the source text again (CachedAccess::load_program,
+    // session/context.rs:158-180); entries point into `jit`, which owns the modules
+    std::unordered_map<std::string, sg_map_entry> map_by_signature;
     // stream capture (sg_graph_begin .. sg_graph_end): blocks allocated AND freed inside the captured
     // region are workspaces whose addresses are baked into the graph; they stay live with the graph
     bool capturing = false;

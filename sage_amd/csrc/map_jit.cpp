@@ -344,8 +344,8 @@ extern "C" int sg_map_compile_only(const char *source, char *log_buf, uint64_t l
     return ok ? SG_OK : SG_ERR_DEVICE;
 }
 
-static int map_prepare(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_tensor *in, int n_in,
-                       const sg_tensor *out, bool need_ptrs, MapPlan &pl, std::string &src, int *res_dt) {
+// Argument checks shared by sg_map and sg_map_source (no text is generated here).
+static int map_check(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_tensor *in, int n_in, const sg_tensor *out, bool need_ptrs) {
     if (!prog || n_prog <= 0 || n_prog > SG_MAX_EXPR) return sg_fail(ctx, SG_ERR_ARG, "sg_map: bad program length %d", n_prog);
     if (n_in < 0 || n_in > SG_MAX_MAP_INPUTS) return sg_fail(ctx, SG_ERR_ARG, "sg_map: %d inputs (max %d)", n_in, SG_MAX_MAP_INPUTS);
     if (n_in && !in) return sg_fail(ctx, SG_ERR_ARG, "sg_map: null inputs");
@@ -369,6 +369,12 @@ static int map_prepare(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_te
                 return sg_fail(ctx, SG_ERR_SHAPE, "sg_map: input %d extent[%d] = %lld, output has %lld (ops.rs:174)", k, a,
                                (long long)in[k].extents[a], (long long)out->extents[a]);
     }
+    return SG_OK;
+}
+
+// Expression text and result dtype (the dtype rules of map.rs:464-501 are enforced while emitting), then the kernel text.
+static int map_generate(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_tensor *in, int n_in, const sg_tensor *out,
+                        const MapPlan &pl, std::string &src, int *res_dt) {
     Gen g{prog, n_prog, in, n_in};
     std::string expr;
     int dt = g.emit(expr);
@@ -377,9 +383,30 @@ static int map_prepare(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_te
     if (res_dt) *res_dt = dt;
     if (dt != out->dtype)
         return sg_fail(ctx, SG_ERR_DTYPE, "sg_map: expression yields dtype %d, output tensor is %d (map.rs:464-501)", dt, out->dtype);
-    plan_map(in, n_in, out, pl);
     src = gen_source(expr, in, n_in, out->dtype, pl);
     return SG_OK;
+}
+
+static int map_prepare(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_tensor *in, int n_in,
+                       const sg_tensor *out, bool need_ptrs, MapPlan &pl, std::string &src, int *res_dt) {
+    int rc = map_check(ctx, prog, n_prog, in, n_in, out, need_ptrs);
+    if (rc != SG_OK) return rc;
+    plan_map(in, n_in, out, pl);
+    return map_generate(ctx, prog, n_prog, in, n_in, out, pl, src, res_dt);
+}
+
+// Everything the generated text depends on, packed into a few dozen bytes: the expression program, the operand
+// dtypes and, per operand, the layout class the plan assigned (extents and strides themselves are kernel arguments).
+static void map_signature(const sg_expr *prog, int n_prog, const sg_tensor *in, int n_in, const MapPlan &pl, std::string &key) {
+    key.clear();
+    key.reserve(16 * (size_t)n_prog + 4 * (size_t)n_in + 8);
+    key.append(reinterpret_cast<const char *>(prog), sizeof(sg_expr) * (size_t)n_prog);
+    const char head[4] = {(char)n_in, (char)pl.ndim, (char)pl.vec, (char)((pl.stream ? 1 : 0) | (pl.need_coords ? 2 : 0))};
+    key.append(head, 4);
+    for (int k = 0; k < n_in; ++k) {
+        const char op[3] = {(char)in[k].dtype, (char)(pl.direct[k] ? 1 : 0), pl.inner[k]};
+        key.append(op, 3);
+    }
 }
 
 extern "C" int sg_map_source(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_tensor *in, int n_in,
@@ -402,17 +429,32 @@ extern "C" int sg_map(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_ten
                       const sg_tensor *out) {
     if (!ctx) return SG_ERR_ARG;
     MapPlan pl;
-    std::string src;
-    int rc = map_prepare(ctx, prog, n_prog, in, n_in, out, true, pl, src, nullptr);
+    int rc = map_check(ctx, prog, n_prog, in, n_in, out, true);
     if (rc != SG_OK) return rc;
+    plan_map(in, n_in, out, pl);
 
-    auto it = ctx->jit.find(src);
-    if (it == ctx->jit.end()) {
-        sg_jit_kernel k{};
-        rc = build_kernel(ctx, src, &k);
+    // A repeat call of an operator finds its kernel by signature; only a new signature generates the kernel text,
+    // and only a new text is built (two signatures may give the same text: the text never mentions literals' provenance).
+    std::string key;
+    map_signature(prog, n_prog, in, n_in, pl, key);
+    auto hit = ctx->map_by_signature.find(key);
+    if (hit == ctx->map_by_signature.end()) {
+        std::string src;
+        int dt = 0;
+        rc = map_generate(ctx, prog, n_prog, in, n_in, out, pl, src, &dt);
         if (rc != SG_OK) return rc;
-        it = ctx->jit.emplace(src, k).first;
+        auto it = ctx->jit.find(src);
+        if (it == ctx->jit.end()) {
+            sg_jit_kernel k{};
+            rc = build_kernel(ctx, src, &k);
+            if (rc != SG_OK) return rc;
+            it = ctx->jit.emplace(src, k).first;
+        }
+        hit = ctx->map_by_signature.emplace(key, sg_map_entry{it->second.fn, dt}).first;
+    } else if (hit->second.result_dtype != out->dtype) {
+        return sg_fail(ctx, SG_ERR_DTYPE, "sg_map: expression yields dtype %d, output tensor is %d (map.rs:464-501)", hit->second.result_dtype, out->dtype);
     }
+    const hipFunction_t fn = hit->second.fn;
 
     // kernel parameter block: layout must match `struct MapParams` in the generated source
     const int nd = pl.ndim, K = n_in > 0 ? n_in : 1;
@@ -443,6 +485,6 @@ extern "C" int sg_map(sg_ctx *ctx, const sg_expr *prog, int n_prog, const sg_ten
     args.push_back(&ptrs[n_in]);
     args.push_back(params.data());
     const unsigned grid = (unsigned)((total + 255) / 256);
-    SG_HIP(ctx, hipModuleLaunchKernel(it->second.fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr));
+    SG_HIP(ctx, hipModuleLaunchKernel(fn, grid, 1, 1, 256, 1, 1, 0, ctx->stream, args.data(), nullptr));
     return SG_OK;
 }

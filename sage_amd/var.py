@@ -773,6 +773,79 @@ def _allow_depth(targets):
         sys.setrecursionlimit(need)
 
 
+def _category(v):
+    """Operator::cat (ops.rs:219-227): maps, Expand (the only Layout, core.rs:319-321), Gemm/GemmBatched
+    (Contract, gemm.rs:166, 328), reduce (reduce.rs:327); everything else keeps the trait default, Other
+    (ops.rs:86-88).  The fused nodes this front-end adds stand for chains containing reductions or products."""
+    if v.op in MAP_OPS:
+        return "map"
+    if v.op == "expand":
+        return "layout"
+    if v.op in GEMM_OPS:
+        return "contract"
+    if v.op == "reduce":
+        return "reduce"
+    return "other"
+
+
+def state_partition(targets, inputs=(), decide_only=False):
+    """Phase 1 of Program::compile (session.rs:101-169): which nodes are STATES, i.e. evaluated once and
+    retained; every other node is recomputed inside each routine that needs it.  Candidates are the operator
+    nodes with two or more consumers plus the outputs, visited in topological order; a candidate's ancestry
+    is walked up to data, earlier states and the program inputs, counting every visited node (a node reached
+    twice counts twice: the walk is over the expanded tree) and collecting the distinct leaves.  It is a state
+    if it is an output, if a Contract / Reduce / Other operator lies on the way, or if nodes x leaves > THRES.
+    Returns {id(state): set of ids of its routine's inputs}; with decide_only the walk stops as soon as the
+    answer is known and the input sets are left incomplete."""
+    targets = list(targets)
+    input_ids = {id(v) for v in inputs}
+    target_ids = {id(t) for t in targets}
+
+    def is_op(v):
+        return v.value is None and v.op != "data"
+
+    nodes, order, stack = {}, {}, [(t, False) for t in targets]
+    while stack:  # reachable nodes and their depth (a topological order)
+        v, expanded = stack.pop()
+        if expanded:
+            order[id(v)] = 1 + max((order[id(i)] for i in v.inputs), default=0) if is_op(v) and id(v) not in input_ids else 0
+            continue
+        if id(v) in nodes:
+            continue
+        nodes[id(v)] = v
+        stack.append((v, True))
+        if is_op(v) and id(v) not in input_ids:
+            stack.extend((i, False) for i in v.inputs)
+    edges = {}
+    for v in nodes.values():
+        if is_op(v) and id(v) not in input_ids:
+            for i in v.inputs:
+                edges[id(i)] = edges.get(id(i), 0) + 1
+    cand = [nodes[k] for k, n in edges.items() if n >= 2 and is_op(nodes[k]) and k not in input_ids and k not in target_ids]
+    cand += targets
+    cand.sort(key=lambda v: order[id(v)])
+    states = {}
+    for node in cand:
+        if id(node) in states:
+            continue
+        leaves, num_ops, complex_op, stack = set(), 0, False, [node]
+        is_target = id(node) in target_ids
+        while stack:
+            v = stack.pop()
+            num_ops += 1
+            if not is_op(v) or id(v) in states or id(v) in input_ids:
+                leaves.add(id(v))
+            else:
+                stack.extend(v.inputs)
+                if _category(v) in ("contract", "reduce", "other"):
+                    complex_op = True
+            if decide_only and (is_target or complex_op or (leaves and num_ops > THRES)):
+                break
+        if is_target or complex_op or num_ops * len(leaves) > THRES:
+            states[id(node)] = leaves
+    return states
+
+
 def _merge_common_subgraphs(targets):
     """Structurally identical operations on the same inputs are computed once: inputs of every node are
     re-pointed at the first node seen with the same (operator, attributes, inputs).  BERT rebuilds the
@@ -812,6 +885,8 @@ class _Evaluator:
         self.targets = {id(t) for t in targets}
         if _FUSION["on"]:
             _merge_common_subgraphs(targets)
+        # which shared nodes are stored once and which are recomputed in every consumer (session.rs:101-169)
+        self.states = state_partition(targets, decide_only=True) if _FUSION["on"] else {}
         _allow_depth(targets)
         seen = set()
         stack = list(targets)
@@ -975,23 +1050,13 @@ class _Evaluator:
         return x.with_shape(x.shape.select_range(a["start"], a["end"] - 1, a["axis"]))
 
     # ---- maps
-    def small(self, v):
-        """session.rs:157-169: a shared node is recomputed in each consumer rather than stored when
-        its un-stored ancestry holds only maps and num_ops * num_inputs <= THRES."""
-        ops, inputs, stack = 0, set(), [v]
-        while stack:
-            n = stack.pop()
-            ops += 1
-            if self.done(n) or n.op not in MAP_OPS:
-                inputs.add(id(n))
-                continue
-            stack.extend(n.inputs)
-        return ops * len(inputs) <= THRES
-
     def inline_ok(self, c):
+        """A map operand is computed inside its consumer's kernel (Operator::fuse, ops.rs:104-161) when the
+        consumer is its only one, or when the reference would not retain it either: a shared node that is no
+        state is recomputed by every routine that reaches it (session.rs:157-169, 524-535)."""
         if not _FUSION["on"] or c.op not in MAP_OPS or self.done(c) or id(c) in self.targets:
             return False
-        return self.n_users(c) <= 1 or self.small(c)
+        return self.n_users(c) <= 1 or id(c) not in self.states
 
     def inline_size(self, v, cap):
         """Program elements v would add if it and everything below it were inlined (capped)."""

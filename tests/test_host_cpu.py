@@ -294,3 +294,102 @@ def test_unseeded_random_nodes_are_never_merged():
     z = c + d
     V._merge_common_subgraphs([z])
     assert z.inputs[0] is z.inputs[1]
+
+
+# ------------------------------------------------------------------ state partition of Program::compile
+class _DryLib:
+    """Stands in for the C-ABI library on a machine without a GPU: allocations hand out fake addresses,
+    every other entry point reports success.  Only the evaluator's decisions are observed, no values."""
+
+    def __init__(self):
+        self.next = 0x10000
+
+    def sg_alloc(self, handle, nbytes, pref):
+        pref._obj.value = self.next
+        self.next += (int(nbytes) + 255) // 256 * 256
+        return 0
+
+    def __getattr__(self, name):
+        return lambda *a: 0
+
+
+class _DryCtx:
+    def __init__(self):
+        self._lib, self.handle, self.launches = _DryLib(), 1, 0
+
+    def check(self, rc):
+        assert rc == 0
+
+
+def _data(ctx, *shape):
+    import sage_amd as S
+    return S.Var.new(S.Tensor.from_numpy(ctx, np.zeros(shape, np.float32)))
+
+
+def test_state_partition_follows_program_compile():
+    """Phase 1 of Program::compile (session.rs:101-169), worked by hand on four small graphs: candidates are the
+    operator nodes with two or more consumers plus the outputs; a candidate is a state if it is an output, if a
+    Contract / Reduce / Other operator lies between it and its leaves (data and earlier states), or if
+    (visited nodes, leaves included) x (distinct leaves) > 5.  The evaluator must store exactly the shared map
+    nodes that are states and recompute the others inside each consumer."""
+    from sage_amd import nn
+    from sage_amd import var as V
+    ctx = _DryCtx()
+
+    def run(targets):
+        ev = V._Evaluator(ctx, targets)
+        for t in targets:
+            ev.get(t)
+        return ev
+
+    # 1. softmax cross-entropy as nn.rs:58-82 composes it.  c = max(x) has two consumers (x - c and log(..) + c)
+    #    and is a reduce: state.  Nothing else is shared.  States: c and the output.
+    x, lab = _data(ctx, 6, 10), V.Var.new(__import__("sage_amd").Tensor.from_numpy(ctx, np.zeros((6, 1), np.uint32)))
+    V.set_fusion(True)
+    c = x.max([1], True)
+    lse = (x - c).exp().sum([1], True).log() + c
+    loss = -((x - lse).gather(lab, 1).sum(1, False))
+    st = V.state_partition([loss])
+    assert set(st) == {id(c), id(loss)}
+    assert st[id(c)] == {id(x)}                      # walk: c, x -> 2 nodes x 1 leaf, but a Reduce lies on the way
+    assert st[id(loss)] == {id(x), id(c), id(lab)}   # the output's routine reads the data and the earlier state
+
+    # 2. layer_norm as nn.rs:84-100 composes it.  mean(x) is built twice (reduce.rs:73-82); identical subgraphs are
+    #    evaluated once here, so the merged mean = sum(x) / n has two consumers (x - mean and mean^2): a map node
+    #    with a Reduce in its ancestry -> state, stored once rather than re-divided in both consumers.
+    x = _data(ctx, 8, 16)
+    g, b = _data(ctx, 1), _data(ctx, 1)
+    y = nn.layer_norm_composed(x, [1], g, b, 1e-5)
+    ev = run([y])
+    shared_maps = [v for v in ev.keep.values() if v.op in V.MAP_OPS and ev.n_users(v) >= 2]
+    mean_nodes = [v for v in shared_maps if v.op == "binary" and v.attrs["name"] == "div" and v.inputs[0].op == "reduce"]
+    assert len(mean_nodes) == 1 and id(mean_nodes[0]) in ev.states and id(mean_nodes[0]) in ev.computed
+
+    # 3. Dense + residual: h = x.W + b feeds a second Dense and the residual addition.  h is a map (the bias
+    #    addition) over a Contract: state.  out = h.W2 + h is the output.
+    x, w, bias, w2 = _data(ctx, 32, 16), _data(ctx, 16, 16), _data(ctx, 16), _data(ctx, 16, 16)
+    h = x.matmul(w) + bias
+    out = h.matmul(w2) + h
+    st = V.state_partition([out])
+    assert set(st) == {id(h), id(out)}
+    assert st[id(out)] == {id(h), id(w2)}
+    ev = run([out])
+    assert id(h) in ev.computed
+
+    # 4. shared maps without any complex operator: the threshold decides.
+    #    u = -(exp(a + b)): walk u, exp, add, a, b = 5 nodes x 2 leaves = 10 > 5 -> state, stored once.
+    #    w = -a: walk w, a = 2 nodes x 1 leaf = 2 -> no state, recomputed inside both consumers.
+    #    s = a - b: walk s, a, b = 3 x 2 = 6 > 5 -> state.   q = a * a: walk q, a, a = 3 x 1 = 3 -> no state.
+    #    (no two of these expressions share an identical sub-expression, which would be evaluated once and change the counts)
+    a, b2 = _data(ctx, 4, 8), _data(ctx, 4, 8)
+    u = -((a + b2).exp())
+    w_ = -a
+    s_ = a - b2
+    q = a * a
+    outs = [u * a, u + b2, w_ * b2, w_ + b2, s_.exp(), s_.log(), q.exp(), q + b2]
+    st = V.state_partition(outs)
+    assert id(u) in st and id(s_) in st and id(w_) not in st and id(q) not in st
+    assert st[id(u)] == {id(a), id(b2)}
+    ev = run(outs)
+    assert id(u) in ev.computed and id(s_) in ev.computed          # materialised once
+    assert id(w_) not in ev.computed and id(q) not in ev.computed  # fused into each consumer

@@ -210,7 +210,7 @@ def cpu_baseline(variant, batch, seq, rng_seed):
 # --------------------------------------------------------------------------------------------
 # Single-kernel workloads (the other configurations the parity tests cover).  Each rotates over
 # enough distinct buffer sets to exceed the 256 MB Infinity Cache, so the rate is an HBM rate.
-def kernel_workloads(ctx, name, rng):
+def kernel_workloads(ctx, name, rng, elements=None):
     """name -> (list of programs to rotate over, algorithmic bytes per call, flops per call,
     kernel label, spec of the oracle's CPU baseline or None).  Every buffer set is a distinct device
     allocation (so the caches cannot serve the next launch) filled from one host array."""
@@ -256,10 +256,15 @@ def kernel_workloads(ctx, name, rng):
         x = normal(B, Cn)
         progs = programs(lambda i: dev(x).sum(1, True), 20)
         return progs, B * Cn * 4 + B * 4, 0.0, "reduce_row_kernel<0, float, true, false>", None
-    if name == "copy":            # plain copy of 64 Mi floats: the kernel of known size that calibrates FETCH_SIZE / WRITE_SIZE
-        n = 64 << 20
-        progs = programs(lambda i: dev(np.ones(n, np.float32)).copy(), 1)
+    if name == "copy":            # plain copy (64 Mi floats by default): the kernel of known size that calibrates FETCH_SIZE / WRITE_SIZE;
+        n = int(elements) if elements else 64 << 20   # with --elements, the copy that moves as many bytes as another workload (its ceiling)
+        x = np.ones(n, np.float32)
+        nbuf = max(1, min(24, (600 << 20) // (8 * n)))  # enough buffer sets to exceed the 256 MB Infinity Cache
+        progs = programs(lambda i: dev(x).copy(), nbuf)
         return progs, 2 * n * 4, 0.0, "sg_map", None
+    if name == "launch_floor":    # a copy of 1024 floats: what one launch costs in a back-to-back stream when it moves nothing
+        progs = programs(lambda i: dev(np.ones(1024, np.float32)).copy(), 4)
+        return progs, 2 * 1024 * 4, 0.0, "sg_map", None
     if name == "gemm_bias":       # config 2: C = A@B + bias, 4096^3
         M = N = K = 4096
         A, Bm, bias = (dev(rng.uniform(-1, 1, s).astype(np.float32)) for s in ((M, K), (K, N), (N,)))
@@ -298,12 +303,12 @@ def oracle_kernel_baseline(spec, rng):
     return None, None
 
 
-def time_kernel_workload(ctx, name, steps, warmup):
+def time_kernel_workload(ctx, name, steps, warmup, elements=None):
     """Times `steps` launches of one single-kernel workload (after `warmup`) between two HIP events on the
     context's stream, rotating over its buffer sets.  Returns (roofline dict, config dict, oracle spec)."""
     from sage_amd import abi
     lib = abi.lib()
-    progs, bytes_per, flops_per, label, spec = kernel_workloads(ctx, name, np.random.default_rng(1))
+    progs, bytes_per, flops_per, label, spec = kernel_workloads(ctx, name, np.random.default_rng(1), elements)
     launches = len(progs[0].calls)
 
     def ev():
@@ -358,7 +363,7 @@ def hbm_rooflines(ctx, steps=600, warmup=200):
 def run_kernel_workload(a):
     import sage_amd as S
     ctx = S.Context(0)
-    roof, cfg, spec = time_kernel_workload(ctx, a.workload, a.steps, a.warmup)
+    roof, cfg, spec = time_kernel_workload(ctx, a.workload, a.steps, a.warmup, a.elements)
     unit, flops_per, bytes_per = roof["unit"], cfg["flops_per_step"], cfg["algorithmic_bytes_per_step"]
     res = {"metric": f"{a.workload} throughput", "value": roof["achieved"], "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
            "ms_per_step": cfg.pop("wall_ms_per_step"), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
@@ -424,7 +429,7 @@ def run_train_workload(a):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="bert", help="bert (default, the headline metric) | resnet18 | resnet18_train | copy | softmax_ce | map_exp_sub | "
+    ap.add_argument("--workload", default="bert", help="bert (default, the headline metric) | resnet18 | resnet18_train | copy | launch_floor | softmax_ce | map_exp_sub | "
                     "bias_residual | layer_norm | softmax | reduce_sum | gemm_bias")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 30; 2000 for the single-kernel workloads, whose step is microseconds)")
@@ -433,6 +438,7 @@ def main():
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--seq", type=int, default=128)
     ap.add_argument("--layers", type=int, default=12)
+    ap.add_argument("--elements", type=int, default=None, help="copy workload: number of floats copied (default 64 Mi)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-hbm-kernels", action="store_true", help="bert: leave out the roofline_hbm list (the fused map/reduce/row kernels timed after the model)")
     ap.add_argument("--graph", choices=["auto", "on", "off"], default="auto",

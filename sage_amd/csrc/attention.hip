@@ -51,9 +51,10 @@ struct AttnP {
 // through LDS at the end (the exact merge of two online-softmax states).  Work units are half as
 // large, which is what balances a short-sequence launch: B*H*L/32 units of 32 queries x all keys
 // may come to 1.5 per SIMD (b32, 12 heads, s128: 1536 units on 1024 SIMDs), i.e. two rounds with half
-// the chip idle in the second; split in two they are 3 per SIMD.
+// the chip idle in the second; split in two they are 3 per SIMD.  Three wavefronts per SIMD need the kernel
+// within 168 registers (the compiler is told so below; the unsplit kernel keeps 2, at 3 it would spill).
 template <int D, bool SPLIT>
-__global__ void __launch_bounds__(64 * NW) attention_kernel(const AttnP p) {
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(SPLIT ? 3 : 2, SPLIT ? 3 : 2))) attention_kernel(const AttnP p) {
     static_assert(D % 32 == 0 && D <= 64, "head size 32 or 64");
     constexpr int QB = SPLIT ? 64 : 32 * NW;   // queries per workgroup
     constexpr int NKB = SPLIT ? 1 : KB / 32;   // 32-key MFMA blocks a wavefront takes from an LDS block
@@ -337,12 +338,11 @@ extern "C" int sg_attention(sg_ctx *ctx, const sg_tensor *q, const sg_tensor *k,
     p.scale = scale;
     if (nb0 * nb1 > 65535) return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention: more than 65535 (batch x head) pairs");
     // Few workgroups of 128 queries (less than two per compute unit): halving the work units (see the kernel)
-    // balances the SIMDs, at the price of a later start of a compute unit's third workgroup and the merge.
-    // Measured at b32 x 12 heads: 68 against 76 us at 128 x 512 (queries x keys), 39 against 43 at 128 x 256,
-    // 15 against 22 at 64 x 128, equal at 128 x 128, slower when the chip is full anyway.
+    // balances the SIMDs.  The split kernel is held to 168 registers so that three of its workgroups share a
+    // compute unit.  Measured at b32 x 12 heads (queries x keys): 23.1 against 25.0 us at 128 x 128, 37 against
+    // 43 at 128 x 256, 63.5 against 76 at 128 x 512, 15 against 22 at 64 x 128; slower once the chip is full anyway.
     const int64_t wgs128 = nb0 * nb1 * ((Lq + 127) / 128);
-    const int64_t tail = Lq % 128;
-    bool split = wgs128 < 2 * (int64_t)(ctx->num_cus > 0 ? ctx->num_cus : 256) && (Lk >= 256 || (tail >= 1 && tail <= 64));
+    bool split = wgs128 < 2 * (int64_t)(ctx->num_cus > 0 ? ctx->num_cus : 256);
     if (const char *e = getenv("SAGE_ATTENTION_SPLIT")) split = atoi(e) != 0;
     const int qb = split ? 64 : 128;
     dim3 grid((unsigned)((Lq + qb - 1) / qb), (unsigned)(nb0 * nb1));

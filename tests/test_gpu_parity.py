@@ -867,6 +867,31 @@ def test_softmax_cross_entropy_rows_far_below_zero(ctx):
     close(yf[16:], ref[16:], REL_MAP, "fused vs float64")
 
 
+def test_softmax_rows_far_below_zero(ctx):
+    """The same for the softmax row kernel, whose exponentials come from the hardware exp2 (results under 2^-126
+    flushed to zero): a row entirely below -87 keeps the shift 0 (reduce.rs:282), every term is denormal, and the
+    kernel redoes the row with the exact routine instead of dividing zero by zero.  Mixed and ordinary rows and a
+    row with a masked half (the attention mask's -1e5) ride along; every row still sums to one."""
+    say("softmax far below zero")
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((48, 128)).astype(np.float32)
+    x[:16] = rng.uniform(-101.0, -89.0, (16, 128)).astype(np.float32)     # every term denormal
+    x[16:32] = rng.uniform(-95.0, -80.0, (16, 128)).astype(np.float32)    # denormal and normal terms mixed
+    add = np.zeros((48, 128), np.float32)
+    add[40:, 64:] = -1e5
+    yf = nn.softmax(dev(ctx, x) + dev(ctx, add), 1).eval(ctx).numpy()
+    yo = O.softmax(O.binary("add", ht(x), ht(add)), [1]).numpy()
+    x64 = (x + add).astype(np.float64)
+    e = np.exp(x64 - np.maximum(x64.max(1, keepdims=True), 0.0))
+    ref = e / e.sum(1, keepdims=True)
+    assert np.all(np.isfinite(yf)) and np.all(np.isfinite(yo))
+    assert np.max(np.abs(yf[:16] - ref[:16])) < 2e-3 and np.max(np.abs(yf[:16] - yo[:16])) < 2e-3   # few bits in denormal terms
+    close(yf[16:], yo[16:], REL_MAP, "fused vs oracle")
+    close(yf[16:], ref[16:], REL_MAP, "fused vs float64")
+    close(yf.sum(1), np.ones(48), 1e-2, "rows sum to one")
+    assert np.all(yf[40:, 64:] == 0.0)
+
+
 @pytest.mark.parametrize("shape,per_feature", [((8, 16, 768), False), ((8, 16, 768), True), ((5, 100), False), ((3, 2050), True), ((64, 64), True)])
 def test_layer_norm(ctx, shape, per_feature):
     say("layer_norm", shape, per_feature)

@@ -183,6 +183,41 @@ def run_timed(ctx, prog, timed):
             ctx.check(rc)
 
 
+def opencl_cpu_devices():
+    """How many CPU devices the installed OpenCL platforms offer (the reference runs on whatever OpenCL device it
+    finds, session/device.rs:36-70; a CPU OpenCL device, e.g. PoCL, would run its own kernels on the host cores).
+    Returns (count, description); (0, why) when there is no loader, no platform or no CPU device."""
+    try:
+        cl = C.CDLL("libOpenCL.so.1")
+    except OSError:
+        return 0, "no OpenCL loader"
+    n = C.c_uint(0)
+    if cl.clGetPlatformIDs(0, None, C.byref(n)) != 0 or n.value == 0:
+        return 0, "OpenCL loader present, no platform"
+    plats = (C.c_void_p * n.value)()
+    cl.clGetPlatformIDs(n.value, plats, None)
+    CL_DEVICE_TYPE_CPU, CL_PLATFORM_NAME = C.c_ulong(1 << 1), 0x0902
+    total, names = 0, []
+    for p in plats:
+        buf = C.create_string_buffer(256)
+        cl.clGetPlatformInfo(C.c_void_p(p), CL_PLATFORM_NAME, 256, buf, None)
+        nd = C.c_uint(0)
+        rc = cl.clGetDeviceIDs(C.c_void_p(p), CL_DEVICE_TYPE_CPU, 0, None, C.byref(nd))
+        names.append(f"{buf.value.decode(errors='replace')}: {nd.value if rc == 0 else 0} CPU devices")
+        total += nd.value if rc == 0 else 0
+    return total, "; ".join(names)
+
+
+def cpu_baseline_kind(entry):
+    """The CPU leg is the oracle (a C port of the reference's kernels).  The reference itself needs a Rust nightly
+    toolchain to build and an OpenCL device to run; the probe records whether the box would at least have offered
+    a CPU OpenCL device to it."""
+    n, what = opencl_cpu_devices()
+    entry["opencl_cpu_devices"] = n
+    entry["opencl_probe"] = what
+    return entry
+
+
 def cpu_baseline(variant, batch, seq, rng_seed):
     """The CPU oracle (oracle/: C restatement of the reference kernels, OpenMP over work-items) on one
     of the 12 encoder layers (whole batch at b32 x s128; at most 4096 tokens of it for larger shapes);
@@ -203,8 +238,8 @@ def cpu_baseline(variant, batch, seq, rng_seed):
     t0 = time.perf_counter()
     O.bert_layer(x, mask, p, heads, act, eps)
     dt = time.perf_counter() - t0
-    return {"value": batch / (12.0 * dt), "unit": "seqs/s", "cores": O.num_threads(), "kind": "port",
-            "sample": f"1 of 12 encoder layers at b{batch} s{seq} in {dt:.2f} s, x12 (embedding and classifier left out)"}
+    return cpu_baseline_kind({"value": batch / (12.0 * dt), "unit": "seqs/s", "cores": O.num_threads(), "kind": "port",
+                              "sample": f"1 of 12 encoder layers at b{batch} s{seq} in {dt:.2f} s, x12 (embedding and classifier left out)"})
 
 
 # --------------------------------------------------------------------------------------------
@@ -348,7 +383,7 @@ def time_kernel_workload(ctx, name, steps, warmup, elements=None):
 HBM_WORKLOADS = ("softmax_ce", "reduce_sum", "map_exp_sub", "softmax", "bias_residual", "layer_norm")
 
 
-def hbm_rooflines(ctx, steps=600, warmup=200):
+def hbm_rooflines(ctx, steps=2000, warmup=500):
     """One roofline entry per fused HBM-bound kernel, each timed back to back on rotating buffer sets."""
     out = []
     for name in HBM_WORKLOADS:

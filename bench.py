@@ -139,7 +139,8 @@ def gemm_calls(ctx, prog):
             M, N, K = c.extents[0] * c.extents[1] * c.extents[2], c.extents[3], f.extents[0] * f.extents[1] * f.extents[2]
             buf = C.create_string_buffer(128)
             ctx.check(lib.sg_gemm_kernel_name(ctx.handle, M, N, K, 1, 1, 1, buf, 128))
-            out.append((i, buf.value.decode().replace(">", ", true>").replace("false, true>", "true, true>"), 2.0 * M * N * K + M * N, (M, N, K, 1)))
+            name = buf.value.decode().rsplit(",", 2)[0] + ", true, true>"  # guarded loads, A read from the image
+            out.append((i, name, 2.0 * M * N * K + M * N, (M, N, K, 1)))
             continue
         if fn in (lib.sg_gemm, lib.sg_gemm_batched, lib.sg_matmul_strided):
             if fn is lib.sg_matmul_strided:
@@ -304,7 +305,7 @@ def kernel_workloads(ctx, name, rng, elements=None):
         M = N = K = 4096
         A, Bm, bias = (dev(rng.uniform(-1, 1, s).astype(np.float32)) for s in ((M, K), (K, N), (N,)))
         progs = programs(lambda i: A.matmul(Bm) + bias, 2)
-        return progs, 4.0 * (M * K + K * N + M * N + N), 2.0 * M * N * K + M * N, "gemm_mfma_kernel<128, 128, 2, true, true, false>", ("gemm", M, N, K)
+        return progs, 4.0 * (M * K + K * N + M * N + N), 2.0 * M * N * K + M * N, "gemm_mfma_kernel<128, 128, 2, true, true, false, false>", ("gemm", M, N, K)
     raise SystemExit(f"unknown workload {name}")
 
 

@@ -882,7 +882,8 @@ extern "C" int sg_gemm_kernel_name(sg_ctx *ctx, int64_t M, int64_t N, int64_t K,
     const TileCfg &t = kTileCfgs[choose_tile(ctx->num_cus, (int)M, (int)N, (int)batch)];
     // the fast instantiation when the shape tiles exactly (operands assumed 16-byte aligned here)
     const bool guard = M % t.bm != 0 || N % t.bn != 0 || K % (2 * BK) != 0;
-    snprintf(buf, cap, "gemm_mfma_kernel<%d, %d, %d, %s, %s, %s>", t.bm, t.bn, t.waves_m, a_k_contiguous ? "true" : "false",
+    // (the last argument is the image-addressed A operand of sg_conv2d, which always takes the guarded instantiation)
+    snprintf(buf, cap, "gemm_mfma_kernel<%d, %d, %d, %s, %s, %s, false>", t.bm, t.bn, t.waves_m, a_k_contiguous ? "true" : "false",
              b_n_contiguous ? "true" : "false", guard ? "true" : "false");
     return SG_OK;
 }

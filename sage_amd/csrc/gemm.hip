@@ -66,6 +66,10 @@ struct ConvG {
     int sh, sw, ph, pw, dh, dw;
     sg_fastdiv d_ohw, d_ow, d_c, d_kw;
     int vec;                       // C % 4 == 0 and the image is 16-byte aligned: four channels per load
+    int fast;                      // C % 16 == 0, at most 64 taps, the image below 2^31 bytes: a slab of 16 k is 16 channels
+                                   // of ONE tap, so unguarded instantiations can fetch A with buffer loads (see the kernel)
+    int ntaps;                     // KH * KW
+    uint32_t img_bytes;            // size of the whole image tensor (fast path only)
 };
 
 struct GemmP {
@@ -232,7 +236,7 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, sg_fastdiv d) { return (__u
 
 template <int BM, int BN, int WAVES_M, bool A_KC, bool B_NC, bool GUARD, bool CONV = false>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3, 8))) gemm_mfma_kernel(const GemmP p) {
-    static_assert(!CONV || (A_KC && GUARD), "the image-addressed A operand is k-contiguous and goes through the guarded loads");
+    static_assert(!CONV || A_KC, "the image-addressed A operand is k-contiguous");
     constexpr int WAVES_N = 4 / WAVES_M;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -328,6 +332,45 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
             cv_k[i] = k_begin + k;
         }
     }
+    // CONV without guards (every tile inside the matrices, C % 16 == 0): a slab of 16 k is 16 consecutive channels of
+    // ONE filter tap, so an item's address is (its output pixel's window origin + its column: fixed for the kernel, a
+    // per-lane 32-bit offset) + (the tap's displacement and the slab's first channel: the same for every lane, a scalar
+    // offset) -- the shape of the plain unguarded loads, served by the same buffer-load instruction.  What the image's
+    // border adds is one bit per item and tap (is this tap of this pixel's window inside the image?), worked out before
+    // the loop; an item whose tap is outside asks for an offset beyond the descriptor's range and receives zeros.
+    // Offsets count from `ph` rows and `pw` pixels before the image, which keeps every per-lane offset non-negative.
+    uint32_t cf_off[TA::NV];
+    uint64_t cf_mask[TA::NV];
+    __amdgpu_buffer_rsrc_t cf_img = a_tile;
+    if (CONV && !GUARD) {
+        const uint32_t lead = ((uint32_t)p.conv.ph * p.conv.W + p.conv.pw) * p.conv.C;  // elements in front of the image
+        cf_img = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.A) - lead, 0, (int)(p.conv.img_bytes + lead * 4u), 0x00020000);
+#pragma unroll
+        for (int i = 0; i < TA::NV; ++i) {
+            int row, k;
+            TA::where(TA::slot(tid + i * NTHREADS), row, k);
+            const uint32_t m = (uint32_t)(m0 + row);
+            const uint32_t n_img = fdiv(m, p.conv.d_ohw), r = m - n_img * (uint32_t)p.conv.ohw;
+            const uint32_t oh = fdiv(r, p.conv.d_ow), ow = r - oh * (uint32_t)p.conv.OW;
+            const int ih0 = (int)oh * p.conv.sh - p.conv.ph, iw0 = (int)ow * p.conv.sw - p.conv.pw;
+            cf_off[i] = (uint32_t)(((n_img * (uint32_t)p.conv.H + (uint32_t)(ih0 + p.conv.ph)) * (uint32_t)p.conv.W + (uint32_t)(iw0 + p.conv.pw)) * (uint32_t)p.conv.C + (uint32_t)k) * 4u;
+            uint64_t mask = 0;
+            for (int t = 0; t < p.conv.ntaps; ++t) {
+                const int ky = t / p.conv.KW, kx = t - ky * p.conv.KW;
+                const int ih = ih0 + ky * p.conv.dh, iw = iw0 + kx * p.conv.dw;
+                if ((unsigned)ih < (unsigned)p.conv.H && (unsigned)iw < (unsigned)p.conv.W) mask |= 1ull << t;
+            }
+            cf_mask[i] = mask;
+        }
+    }
+    auto conv_fast = [&](f32x4 &r, int i, int k0) {
+        const uint32_t kb = (uint32_t)(k_begin + k0);  // the same for every lane: scalar arithmetic
+        const uint32_t tap = fdiv(kb, p.conv.d_c), c0 = kb - tap * (uint32_t)p.conv.C;
+        const uint32_t ky = fdiv(tap, p.conv.d_kw), kx = tap - ky * (uint32_t)p.conv.KW;
+        const uint32_t slab_off = ((ky * (uint32_t)p.conv.dh * (uint32_t)p.conv.W + kx * (uint32_t)p.conv.dw) * (uint32_t)p.conv.C + c0) * 4u;
+        const uint32_t lane_off = ((cf_mask[i] >> tap) & 1ull) ? cf_off[i] : 0x80000000u;
+        TA::load_one_fast(r, cf_img, lane_off, slab_off);
+    };
     auto conv_load = [&](f32x4 &r, int i, int k0) {
         f32x4 v = {0.f, 0.f, 0.f, 0.f};
         const int gk = cv_k[i] + k0, k_lim = k_begin + Kloc;
@@ -358,7 +401,8 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     do {                                                                                       \
         if ((e) < TA::NV) {                                                                    \
             const int ia = (e) < TA::NV ? (e) : 0;                                         \
-            if (CONV) conv_load(RA[ia], ia, (k0));                                             \
+            if (CONV && GUARD) conv_load(RA[ia], ia, (k0));                                    \
+            else if (CONV) conv_fast(RA[ia], ia, (k0));                                        \
             else if (GUARD) TA::load_one_guarded(RA[ia], ia, A, m0, (k0), p.M, Kloc, p.a_sm, p.a_sk, p.vec_a, tid); \
             else TA::load_one_fast(RA[ia], a_tile, off_a[ia], TA::slab_offset((k0), (uint32_t)p.a_sk)); \
         } else {                                                                               \
@@ -638,7 +682,7 @@ template <int BM, int BN, int WAVES_M, bool GUARD>
 void launch_layouts(sg_ctx *ctx, const GemmP &p, dim3 grid, bool a_kc, bool b_nc) {
     dim3 block(NTHREADS);
     if (p.conv.ohw) {  // image-addressed A (sg_conv2d): one instantiation per tile shape
-        if constexpr (GUARD) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, true, true>), grid, block, 0, ctx->stream, p);
+        hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD, true>), grid, block, 0, ctx->stream, p);
         return;
     }
     if (a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD>), grid, block, 0, ctx->stream, p);
@@ -655,14 +699,15 @@ bool needs_guard(const GemmP &p, int bm, int bn, bool a_kc, bool b_nc) {
     const int64_t reach_b = b_nc ? (int64_t)p.K * p.b_sk + bn : (int64_t)bn * p.b_sn + p.K;
     const bool fits32 = reach_a >= 0 && reach_b >= 0 && reach_a < (1ll << 29) && reach_b < (1ll << 29);
     const bool vec_out = p.vec_c && (!p.res || p.vec_r) && (!p.bias || p.vec_bias);
-    if (p.conv.ohw) return true;
+    // image-addressed A: unguarded when the slabs are single taps (conv.fast) and B, C and the tiling allow it
+    if (p.conv.ohw) return !p.conv.fast || p.M % bm != 0 || p.N % bn != 0 || p.K % (2 * BK) != 0 || !p.vec_b || !vec_out || reach_b < 0 || reach_b >= (1ll << 29);
     return p.M % bm != 0 || p.N % bn != 0 || p.K % (2 * BK) != 0 || !p.vec_a || !p.vec_b || !vec_out || !fits32;
 }
 
 // How many k ranges to split into.  Splitting pays when the output has too few tiles to occupy the
 // chip and K is long: each range becomes its own workgroup (grid z) writing a partial product, and a
 // second kernel sums them.  Ranges are multiples of 32 so that the unguarded loop stays legal.
-int choose_split(int num_cus, int64_t wgs, int K, bool image_operand, int *k_chunk) {
+int choose_split(int num_cus, int64_t wgs, int K, bool guarded_image_operand, int *k_chunk) {
     const int64_t cus = num_cus > 0 ? num_cus : 256;
     *k_chunk = 0;
     const char *force = getenv("SAGE_GEMM_SPLITK");
@@ -671,9 +716,8 @@ int choose_split(int num_cus, int64_t wgs, int K, bool image_operand, int *k_chu
     else {
         // One 64x64 tile per compute unit multiplies 16 of k in about 0.21 us; the second pass and the extra launch
         // cost about 11 us more than they save below K = 1024 (measured at 64..98 workgroups, K = 512..1152).
-        // With the A operand read from an image every slab also pays the window arithmetic, and splitting
-        // pays from K = 512 (ResNet-18 forward: 0.365 against 0.398 ms).
-        if (wgs * 2 > cus || K < (image_operand ? 512 : 1024)) return 1;
+        // The guarded image-addressed loads pay the window arithmetic in every slab: there splitting pays from K = 512.
+        if (wgs * 2 > cus || K < (guarded_image_operand ? 512 : 1024)) return 1;
         want = (int)((2 * cus + wgs - 1) / wgs);
         if (want > K / 128) want = K / 128;
         if (want > 32) want = 32;
@@ -718,7 +762,7 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noal
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     int k_chunk = 0;
-    const int nsplit = choose_split(ctx->num_cus, (int64_t)p.tiles_m * p.tiles_n * batch, p.K, p.conv.ohw != 0, &k_chunk);
+    const int nsplit = choose_split(ctx->num_cus, (int64_t)p.tiles_m * p.tiles_n * batch, p.K, p.conv.ohw != 0 && !p.conv.fast, &k_chunk);
     if (nsplit > 1) {
         const int64_t slice = (int64_t)batch * p.M * p.N;
         void *ws = nullptr;
@@ -951,6 +995,10 @@ extern "C" int sg_conv2d(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *filte
     g.d_c = sg_make_fastdiv((uint32_t)Cc); g.d_kw = sg_make_fastdiv((uint32_t)KW);
     const float *img = (const float *)x->base + x->offset;
     g.vec = Cc % 4 == 0 && ptr_aligned16(img);
+    g.ntaps = (int)(KH * KW);
+    const int64_t img_bytes = N * H * W * Cc * 4, lead_bytes = ((int64_t)pad[1] * W + pad[0]) * Cc * 4;
+    g.fast = Cc % 16 == 0 && ptr_aligned16(img) && KH * KW <= 64 && img_bytes + lead_bytes < (1ll << 31);
+    g.img_bytes = g.fast ? (uint32_t)img_bytes : 0u;
     // A = the virtual [M, K] column matrix (row stride K, never dereferenced through it), B = filter as [K, OC], C = out as [M, OC]
     Mat ma{img, 0, 0, K, 1};
     Mat mb{(const float *)filter->base + filter->offset, 0, 0, OC, 1};

@@ -601,6 +601,14 @@ CONV_CASES = [
     (2, 7, 7, 128, 1, 1, 256, [2, 2], [0, 0], [1, 1]),    # 1x1 stride-2 downsample
     (16, 4, 4, 256, 3, 3, 256, [1, 1], [1, 1], [1, 1]),   # few output tiles and K = 2304: split-K
     (1, 6, 6, 4, 3, 3, 8, [1, 1], [1, 1], [0, 0]),        # dilation 0 (every tap reads the window's corner, as the reference would)
+    # exactly tiled outputs with C % 16 == 0: the unguarded instantiation, A fetched with buffer loads, border taps masked
+    (4, 8, 8, 64, 3, 3, 64, [1, 1], [1, 1], [1, 1]),      # M = 256, K = 576
+    (4, 8, 8, 32, 3, 3, 128, [2, 2], [1, 1], [1, 1]),     # stride 2: M = 64, K = 288
+    (2, 16, 8, 16, 7, 7, 64, [1, 1], [3, 3], [1, 1]),     # 49 taps, M = 256, K = 784 (not a multiple of 32: guarded after all)
+    (2, 16, 8, 32, 5, 3, 64, [1, 1], [2, 1], [2, 1]),     # 15 taps, dilation 2 across the width, M = 256, K = 480
+    (8, 4, 4, 128, 1, 1, 64, [2, 2], [0, 0], [1, 1]),     # 1x1 stride 2 downsample: M = 32 ... guarded; and
+    (32, 4, 4, 128, 1, 1, 64, [2, 2], [0, 0], [1, 1]),    # the same at M = 128: unguarded
+    (64, 2, 2, 256, 3, 3, 256, [1, 1], [1, 1], [1, 1]),   # M = 256, K = 2304: unguarded and split-K
 ]
 
 

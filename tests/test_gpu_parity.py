@@ -617,7 +617,7 @@ def test_conv2d_without_column_matrix(ctx, monkeypatch, case):
     """sg_conv2d reads the GEMM's A operand from the image through the im2col window arithmetic.  It must
     equal the oracle's im2col + gemm (conv.rs:61-96) within the GEMM tolerance, and the explicit
     sg_im2col + sg_gemm path bit for bit where both split K the same way (same tiles, same k order; between
-    K = 512 and 1024 only the image-addressed product is split), with and without bias / ReLU / residual."""
+    K = 512 and 1024 the guarded image-addressed product is split and the plain one is not), with and without bias / ReLU / residual."""
     n, h, w, c, kh, kw, oc, stride, pad, dil = case
     say("conv2d", case)
     rng = np.random.default_rng(n * 100 + c)

@@ -557,6 +557,16 @@ def conv_2d(x, filt, stride, pad, dil):  # conv.rs:61-96
     return matmul(col, f).view([n, ch, cw, cout])
 
 
+def conv_transpose_2d(x, filt, stride, pad, dil):  # conv.rs:98-140 (output size: conv.rs:33-45)
+    n, h, w, cin = x.extents
+    kh, kw, cout = filt.extents[0], filt.extents[1], filt.extents[2]
+    f = filt.permute([2, 0, 1, 3]).organize().view([cin, kh * kw * cout])
+    col = matmul(x.view([n * h * w, cin]), f).view([n, h, w, kh, kw, cout])
+    ker, stride, pad, dil = [kw, kh], _pair(stride), _pair(pad), _pair(dil)
+    out = [(s - 1) * st - 2 * p + d * (k - 1) for s, k, st, p, d in zip([w, h], ker, stride, pad, dil)]
+    return col2im(col, out, ker, stride, pad, dil)
+
+
 def max_pool_2d(x, ker, stride, pad, dil):  # conv.rs:155-165
     return rmax(im2col(x, ker, stride, pad, dil), [3, 4], False)
 

@@ -707,7 +707,7 @@ bool needs_guard(const GemmP &p, int bm, int bn, bool a_kc, bool b_nc) {
 // How many k ranges to split into.  Splitting pays when the output has too few tiles to occupy the
 // chip and K is long: each range becomes its own workgroup (grid z) writing a partial product, and a
 // second kernel sums them.  Ranges are multiples of 32 so that the unguarded loop stays legal.
-int choose_split(int num_cus, int64_t wgs, int K, bool guarded_image_operand, int *k_chunk) {
+int choose_split(int num_cus, int64_t wgs, int K, bool guarded_loop, int *k_chunk) {
     const int64_t cus = num_cus > 0 ? num_cus : 256;
     *k_chunk = 0;
     const char *force = getenv("SAGE_GEMM_SPLITK");
@@ -716,8 +716,9 @@ int choose_split(int num_cus, int64_t wgs, int K, bool guarded_image_operand, in
     else {
         // One 64x64 tile per compute unit multiplies 16 of k in about 0.21 us; the second pass and the extra launch
         // cost about 11 us more than they save below K = 1024 (measured at 64..98 workgroups, K = 512..1152).
-        // The guarded image-addressed loads pay the window arithmetic in every slab: there splitting pays from K = 512.
-        if (wgs * 2 > cus || K < (guarded_image_operand ? 512 : 1024)) return 1;
+        // The guarded loads pay bounds checks (and, image-addressed, the window arithmetic) in every slab: there
+        // splitting pays from K = 512.
+        if (wgs * 2 > cus || K < (guarded_loop ? 512 : 1024)) return 1;
         want = (int)((2 * cus + wgs - 1) / wgs);
         if (want > K / 128) want = K / 128;
         if (want > 32) want = 32;
@@ -762,7 +763,7 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noal
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     int k_chunk = 0;
-    const int nsplit = choose_split(ctx->num_cus, (int64_t)p.tiles_m * p.tiles_n * batch, p.K, p.conv.ohw != 0 && !p.conv.fast, &k_chunk);
+    const int nsplit = choose_split(ctx->num_cus, (int64_t)p.tiles_m * p.tiles_n * batch, p.K, needs_guard(p, BM, BN, a_kc, b_nc), &k_chunk);
     if (nsplit > 1) {
         const int64_t slice = (int64_t)batch * p.M * p.N;
         void *ws = nullptr;

@@ -598,6 +598,27 @@ def conv_2d(x, filt, stride, padding, dilation):
     return col.matmul(f).view([n, ch, cw, cout])
 
 
+def conv_transpose_2d(x, filt, stride, padding, dilation):
+    """conv.rs:98-140, as written there: the filter's axis 2 is taken as the output channel count and its
+    permutation (2,0,1,3) is viewed as [C_in, KH*KW*that], so extent 3 must equal x's channels; the product's
+    [N,H,W,KH,KW,OC] columns are folded by col2im onto an image of (size-1)*stride - 2*pad + dil*(ker-1)
+    per side (conv.rs:33-45: one less than the usual transposed-convolution size)."""
+    filt, x = into_var(filt), into_var(x)
+    if filt.rank != 4 or x.rank != 4:
+        raise abi.ShapeError(abi.ERR_SHAPE, "conv_transpose_2d needs x [N,H,W,C] and a rank-4 filter (conv.rs:104-116)")
+    n, h, w, cin = x.extents
+    kh, kw, cout = filt.extents[0], filt.extents[1], filt.extents[2]
+    ker, stride, pad, dil = [kw, kh], _pair(stride), _pair(padding), _pair(dilation)
+    if filt.extents[3] != cin:
+        raise abi.ShapeError(abi.ERR_SHAPE, "conv_transpose_2d: filter does not view as [C_in, KH*KW*OC] (conv.rs:125)")
+    f = filt.permute([2, 0, 1, 3]).organize().view([cin, kh * kw * cout])
+    col = x.view([n * h * w, cin]).matmul(f).view([n, h, w, kh, kw, cout])
+    out = [(s - 1) * st - 2 * p + d * (k - 1) for s, k, st, p, d in zip([w, h], ker, stride, pad, dil)]
+    if min(out) < 1:
+        raise abi.ShapeError(abi.ERR_SHAPE, "conv_transpose_2d: empty output (conv.rs:42)")
+    return col2im(col, out, ker, stride, pad, dil)
+
+
 def avg_pool_2d(x, ker_size, stride, padding, dilation):
     """conv.rs:143-153."""
     return im2col(x, ker_size, stride, padding, dilation).mean([3, 4], False)

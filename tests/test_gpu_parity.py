@@ -592,6 +592,37 @@ def test_conv_and_pools(ctx):
     close(V.avg_pool_2d(dev(ctx, xp), 2, 2, 0, 1).eval(ctx).numpy(), O.avg_pool_2d(ht(xp), 2, 2, 0, 1).numpy(), REL_MAP, "avg_pool")
 
 
+@pytest.mark.parametrize("geom", [((2, 5, 6, 4), (3, 3, 4, 4), 2, 1, 1), ((1, 7, 4, 8), (2, 3, 8, 8), [2, 1], [0, 1], [1, 2]),
+                                  ((1, 7, 4, 8), (2, 3, 8, 8), [1, 2], [1, 0], [2, 2]), ((3, 4, 4, 6), (3, 3, 5, 6), 2, 0, 1), ((2, 6, 6, 16), (4, 4, 16, 16), 2, 1, 1)])
+def test_conv_transpose_2d(ctx, geom):
+    """conv_transpose_2d (conv.rs:98-140) = view -> matmul with the permuted filter -> col2im, onto the
+    reference's output size (conv.rs:33-45, one less per side than the usual formula).  Against the oracle's
+    composition, and, where the filter's two channel extents are equal (the only case in which the reference's
+    view of the filter is a transposition) and both dilations agree (col2im takes the row dilation for both
+    remainders, conv.rs:418-473), against torch's conv_transpose2d cropped to that size."""
+    import torch
+    import torch.nn.functional as F
+    xs, fs, stride, pad, dil = geom
+    say("conv_transpose_2d", geom)
+    rng = np.random.default_rng(sum(xs) + sum(fs))
+    x = rng.standard_normal(xs).astype(np.float32)
+    f = (rng.standard_normal(fs) * 0.3).astype(np.float32)
+    y = V.conv_transpose_2d(dev(ctx, x), dev(ctx, f), stride, pad, dil).eval(ctx).numpy()
+    yo = O.conv_transpose_2d(ht(x), ht(f), stride, pad, dil).numpy()
+    assert y.shape == yo.shape
+    close(y, yo, REL_GEMM, "conv_transpose_2d vs oracle")
+    pr = lambda v: [v, v] if isinstance(v, int) else list(v)  # [w, h] pairs
+    st, pd, dl = pr(stride), pr(pad), pr(dil)
+    if fs[2] == fs[3] and dl[0] == dl[1]:
+        # torch's weight is [C_in, C_out, KH, KW]; the reference contracts x's channels with filter axis 2
+        t = F.conv_transpose2d(torch.from_numpy(x).permute(0, 3, 1, 2).double(), torch.from_numpy(f).permute(2, 3, 0, 1).double(),
+                               stride=(st[1], st[0]), padding=(pd[1], pd[0]), dilation=(dl[1], dl[0])).permute(0, 2, 3, 1).numpy()
+        assert t.shape[1] == y.shape[1] + 1 and t.shape[2] == y.shape[2] + 1
+        close(y, t[:, :y.shape[1], :y.shape[2], :], REL_GEMM, "conv_transpose_2d vs torch")
+    with pytest.raises(abi.ShapeError):
+        V.conv_transpose_2d(dev(ctx, x), dev(ctx, f[:, :, :, :-1].copy()), stride, pad, dil)
+
+
 CONV_CASES = [
     # (n, h, w, c, kh, kw, oc, stride [w,h], pad [w,h], dil [w,h])
     (2, 12, 10, 5, 3, 3, 7, [2, 2], [1, 1], [1, 1]),      # channels not a multiple of 4: scalar taps

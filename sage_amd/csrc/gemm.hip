@@ -714,12 +714,12 @@ int choose_split(int num_cus, int64_t wgs, int K, bool guarded_loop, int *k_chun
     int want;
     if (force) want = atoi(force);
     else {
-        // One 64x64 tile per compute unit multiplies 16 of k in about 0.21 us; the second pass and the extra launch
-        // cost about 11 us more than they save below K = 1024 (measured at 64..98 workgroups, K = 512..1152).
-        // The guarded loads pay bounds checks (and, image-addressed, the window arithmetic) in every slab: there
-        // splitting pays from K = 512.
-        if (wgs * 2 > cus || K < (guarded_loop ? 512 : 1024)) return 1;
-        want = (int)((2 * cus + wgs - 1) / wgs);
+        // The matrix pipe of a compute unit is what a workgroup's loop occupies: two workgroups on one unit take
+        // twice as long as one, so the ranges are cut so that tiles x ranges fills the units ONCE (measured on
+        // 16, 32 and 64 tiles with K = 576..4608: the time has its minimum at tiles x ranges = 256 and jumps by
+        // a quarter right above it).
+        if (wgs * 2 > cus) return 1;
+        want = (int)(cus / wgs);
         if (want > K / 128) want = K / 128;
         if (want > 32) want = 32;
     }
@@ -727,6 +727,9 @@ int choose_split(int num_cus, int64_t wgs, int K, bool guarded_loop, int *k_chun
     int chunk = ((K + want - 1) / want + 31) / 32 * 32;
     const int nsplit = (K + chunk - 1) / chunk;
     if (nsplit < 2) return 1;
+    // A tile multiplies 16 of k in about 0.21 us (more with guarded loads); the second pass and its launch cost
+    // about 5 us: the split has to take that many slabs off a workgroup's loop.
+    if (!force && (K / 16) * (nsplit - 1) / nsplit < (guarded_loop ? 16 : 24)) return 1;
     *k_chunk = chunk;
     return nsplit;
 }

@@ -286,6 +286,25 @@ int sg_col2im(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, const int32
 int sg_rand_uniform(sg_ctx *ctx, uint32_t seed_x, uint32_t seed_y, const sg_tensor *out);
 int sg_rand_normal(sg_ctx *ctx, uint32_t seed_x, uint32_t seed_y, const sg_tensor *out);
 
+/* ---- optimizer step: optim.rs ------------------------------------------------------------------ */
+
+/* Scalars of Adam (optim.rs:98-127).  one_minus_beta1/2 are passed, not derived: the reference forms
+ * 1 - beta in f64 on the host and rounds once when the scalar enters the expression. */
+typedef struct sg_adam_hyper {
+    float lr, beta1, beta2, one_minus_beta1, one_minus_beta2, eps, weight_decay;
+} sg_adam_hyper;
+
+/* Adam::update (optim.rs:129-177) for n_tensors parameters in place, up to 32 per launch: for each i,
+ * values[i], m[i], v[i] are rewritten from grads[i] by the expressions the reference builds out of map
+ * operators (m' = m*beta1 + g*(1-beta1); v' = v*beta2 + pow(g,2)*(1-beta2); value' = value -
+ * (m'/(1-beta1^t))*lr / (sqrt(v'/(1-beta2^t)) + eps); g = grad + value*weight_decay when that is not 0),
+ * operation for operation and uncontracted: bit-identical to evaluating those operators.  step: one fp32
+ * element on the device holding t (the reference keeps t as a tensor, optim.rs:165-176; it is read, not
+ * advanced).  All tensors dense fp32, values[i]/grads[i]/m[i]/v[i] of equal size.  Everything is validated
+ * before the first launch. */
+int sg_adam_update(sg_ctx *ctx, int n_tensors, const sg_tensor *values, const sg_tensor *grads,
+                   const sg_tensor *m, const sg_tensor *v, const sg_tensor *step, const sg_adam_hyper *h);
+
 /* ---- fused row operators: compositions of ops/nn.rs ------------------------------------------ */
 
 /* softmax over the last axis (nn.rs:42-56) of (x + addend): one pass instead of reduce(max),

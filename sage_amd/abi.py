@@ -46,6 +46,11 @@ class sg_gemm_epilogue(C.Structure):
                 ("bias", C.POINTER(sg_tensor)), ("residual", C.POINTER(sg_tensor))]
 
 
+class sg_adam_hyper(C.Structure):
+    _fields_ = [("lr", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float), ("one_minus_beta1", C.c_float),
+                ("one_minus_beta2", C.c_float), ("eps", C.c_float), ("weight_decay", C.c_float)]
+
+
 _TP = C.POINTER(sg_tensor)
 _CTX = C.c_void_p
 _I32P = C.POINTER(C.c_int32)
@@ -99,6 +104,7 @@ PROTOTYPES = {
     "sg_graph_destroy": (C.c_int, [_CTX, C.c_void_p]),
     "sg_rand_uniform": (C.c_int, [_CTX, C.c_uint32, C.c_uint32, _TP]),
     "sg_rand_normal": (C.c_int, [_CTX, C.c_uint32, C.c_uint32, _TP]),
+    "sg_adam_update": (C.c_int, [_CTX, C.c_int, _TP, _TP, _TP, _TP, _TP, C.POINTER(sg_adam_hyper)]),
     "sg_attention": (C.c_int, [_CTX, _TP, _TP, _TP, _TP, C.c_float, _TP]),
 }
 

@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libsage_hip.so")
-SOURCES = ["runtime.cpp", "map_jit.cpp", "reduce.hip", "index.hip", "gemm.hip", "attention.hip", "rand.hip"]
+SOURCES = ["runtime.cpp", "map_jit.cpp", "reduce.hip", "index.hip", "gemm.hip", "attention.hip", "rand.hip", "optim.hip"]
 # -packed-fp32-ops is switched off: hipcc would otherwise form v_pk_*_f32 from plain float code.
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -14,7 +14,8 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Wall", "-Wno-u
 
 # Per-source additions.  attention.hip: accumulators in ordinary vector registers; the compiler's default put
 # the output accumulators into the accumulation file and copied them out and back for every rescaling.
-EXTRA = {"attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+# optim.hip: the fused optimizer step must round like the generated map kernels it stands for (no contraction).
+EXTRA = {"attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"], "optim.hip": ["-ffp-contract=off"]}
 
 
 def build(verbose=True):

@@ -208,9 +208,6 @@ void plan_map(const sg_tensor *in, int n_in, const sg_tensor *out, MapPlan &pl) 
         }
     }
     pl.vec = vec_ok ? 4 : 1;
-    int64_t total = 1;
-    for (int a = 0; a < nd; ++a) total *= ext[a];
-    total /= pl.vec;
     int64_t bytes = sg_numel(out) * 4;
     for (int k = 0; k < n_in; ++k) {
         int64_t distinct = 1;

@@ -85,8 +85,18 @@ __global__ void __launch_bounds__(256) reduce_thread_kernel(const T *__restrict_
     const T *p = x + x_off + decompose(kept, gid);
     T acc = ref_zero ? (T)0 : identity<OP, T>();
     if (red.n == 1) {
-        const uint32_t s = red.stride[0];
-        for (uint32_t i = 0; i < red.ext[0]; ++i) acc = combine<OP, T>(acc, p[i * s]);
+        // eight independent requests at a time, combined in index order: the result is that of the plain loop,
+        // which would wait for each element in turn (128 partial sums: 30 us against 5)
+        const uint32_t s = red.stride[0], n = red.ext[0];
+        uint32_t i = 0;
+        for (; i + 8 <= n; i += 8) {
+            T v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = p[(i + u) * s];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc = combine<OP, T>(acc, v[u]);
+        }
+        for (; i < n; ++i) acc = combine<OP, T>(acc, p[i * s]);
     } else {
         for (uint32_t i = 0; i < red_total; ++i) acc = combine<OP, T>(acc, p[decompose(red, i)]);
     }
@@ -108,7 +118,15 @@ __global__ void __launch_bounds__(256) reduce_cols_kernel(const T *__restrict__ 
     T acc = identity<OP, T>();
     if (c < n_cols) {
         const T *p = x + x_off + c;
-        for (uint32_t r = r0 + ty; r < r1; r += 4) acc = combine<OP, T>(acc, p[(size_t)r * row_stride]);
+        uint32_t r = r0 + ty;
+        for (; r + 12 < r1; r += 16) {  // four rows in flight, combined in row order
+            T v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = p[(size_t)(r + 4 * u) * row_stride];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc = combine<OP, T>(acc, v[u]);
+        }
+        for (; r < r1; r += 4) acc = combine<OP, T>(acc, p[(size_t)r * row_stride]);
     }
     sh[ty][threadIdx.x & 63u] = acc;
     __syncthreads();

@@ -154,11 +154,16 @@ class Adam(Optimizer):
             _assign(param, (param - m_hat * self.lr / (v_hat.sqrt() + self.eps)).eval(ctx), ctx)
         self.t = (t + 1.0).eval(ctx)
 
-    def compile(self, grads, ctx):
+    def compile(self, grads, ctx, fused=True):
+        """fused=True (default, when every tensor is dense fp32): all parameters are updated by sg_adam_update,
+        one launch per 32 of them, followed by t <- t + 1.  fused=False replays the reference's operators: three
+        map kernels and three copies per parameter.  Both give the same bits."""
         if self.t is None or any(id(g) not in self.m_t for g in grads.values()):
             raise RuntimeError("Adam.compile needs the state of every gradient: call update() once first "
                                "(the first update creates all-zero moments, optim.rs:149-163)")
         t = Var.new(self.t)
+        if fused and self._fusable(grads, ctx):
+            return self._compile_fused(grads, ctx, t)
         pairs = []
         for param, grad in grads.items():
             gv = Var.new(_value(grad, ctx))
@@ -172,3 +177,32 @@ class Adam(Optimizer):
                       (param - m_hat * self.lr / (v_hat.sqrt() + self.eps), param.value)]
         pairs.append((t + 1.0, self.t))
         return _compile(ctx, pairs)
+
+    def _fusable(self, grads, ctx):
+        from . import abi
+        for param, grad in grads.items():
+            ts = (param.value, _value(grad, ctx), self.m_t[id(grad)], self.v_t[id(grad)])
+            if any(x is None or x.dtype != abi.FLOAT or not x.is_dense() or x.extents != ts[0].extents for x in ts):
+                return False
+        return True
+
+    def _compile_fused(self, grads, ctx, t):
+        from . import abi
+        lib = ctx._lib
+        n = len(grads)
+        cols = [[], [], [], []]
+        for param, grad in grads.items():
+            for col, x in zip(cols, (param.value, grad.value, self.m_t[id(grad)], self.v_t[id(grad)])):
+                col.append(x)
+        arrays = [(abi.sg_tensor * max(n, 1))(*[x.c() for x in col]) for col in cols]
+        hyper = abi.sg_adam_hyper(self.lr, self.beta1, self.beta2, 1.0 - self.beta1, 1.0 - self.beta2, self.eps, self.weight_decay)
+        step = self.t.c()
+        prog = _compile(ctx, [])
+        args = (C.c_int(n), *arrays, C.byref(step), C.byref(hyper))
+        ctx.check(lib.sg_adam_update(ctx.handle, *args))
+        prog.calls.append((lib.sg_adam_update, args, [cols, arrays, hyper, step, self.t]))
+        # t <- t + 1 behind the update (which reads it)
+        tail = _compile(ctx, [(t + 1.0, self.t)])
+        prog.calls += tail.calls
+        prog.keep = tail
+        return prog

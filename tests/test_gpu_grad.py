@@ -437,3 +437,97 @@ def test_fused_sibling_dense_follows_parameter_updates(ctx):
     p2["wq"] = p["wq"]
     close(prog.run()[0].numpy(), torch_bert_layer(x, mask, p2, heads, "gelu", 1e-12), REL_GEMM, "graph replay after a host write")
     prog.release_graph()
+
+
+ADAM_SHAPES = [(1,), (3,), (5, 7), (64,), (33, 17), (128, 96), (4100,), (2, 3, 4, 5), (1024,), (1025,), (7, 7, 1, 64)] + \
+    [(16 + i,) for i in range(24)] + [(3, 3, 64, 64)]
+
+
+@pytest.mark.parametrize("weight_decay", [0.0, 0.01])
+def test_adam_fused_update_is_the_operator_chain(ctx, weight_decay):
+    """sg_adam_update (all parameters in one or two launches, in place) against Adam::update replayed as the
+    reference's map operators (optim.rs:129-177): bit-identical values, moments and step counter over several
+    steps with changing gradients, eager and as a HIP graph; 36 tensors (two launches), sizes around the
+    4-element and 1024-element boundaries; and against the expressions in float64."""
+    say("adam fused", weight_decay)
+    rng = np.random.default_rng(53)
+    w0 = [rng.standard_normal(s).astype(np.float32) for s in ADAM_SHAPES]
+    g_steps = [[(rng.standard_normal(s) * 0.1).astype(np.float32) for s in ADAM_SHAPES] for _ in range(6)]
+
+    def make():
+        params = [dev(ctx, w) for w in w0]
+        gvars = [dev(ctx, g) for g in g_steps[0]]
+        return params, gvars, dict(zip(params, gvars)), optim.Adam(1e-2, weight_decay=weight_decay)
+
+    def feed(gvars, gs):
+        for gv, g in zip(gvars, gs):
+            gv.value.copy_from_numpy(g)
+
+    pa, ga, grads_a, opt_a = make()
+    pb, gb, grads_b, opt_b = make()
+    w = [x.astype(np.float64) for x in w0]
+    m = [np.zeros_like(x) for x in w]
+    v = [np.zeros_like(x) for x in w]
+    t = 1.0
+
+    def numpy_step(gs, first=False):
+        nonlocal t
+        for i, g in enumerate(gs):
+            g = g.astype(np.float64) + w[i] * weight_decay if weight_decay else g.astype(np.float64)
+            if not first:
+                m[i] = m[i] * 0.9 + g * (1.0 - 0.9)
+                v[i] = v[i] * 0.999 + g ** 2 * (1.0 - 0.999)
+            w[i] = w[i] - (m[i] / (1.0 - 0.9 ** t)) * 1e-2 / (np.sqrt(v[i] / (1.0 - 0.999 ** t)) + 1e-8)
+        t += 1.0
+
+    for step in range(2):  # the first update stores zero moments (optim.rs:149-163), the second accumulates
+        for gv, o in ((ga, opt_a), (gb, opt_b)):
+            feed(gv, g_steps[step])
+        opt_a.update(grads_a, ctx)
+        opt_b.update(grads_b, ctx)
+        numpy_step(g_steps[step], first=step == 0)
+    feed(ga, g_steps[2]); feed(gb, g_steps[2])
+    n0 = ctx.launches
+    prog_a = opt_a.compile(grads_a, ctx)                 # building performs update 3
+    fused_launches = ctx.launches - n0
+    prog_b = opt_b.compile(grads_b, ctx, fused=False)
+    numpy_step(g_steps[2])
+    assert len(prog_a.calls) == 1 + 2, len(prog_a.calls)  # one call (two launches for 36 tensors), t + 1 and its copy
+    assert len(prog_b.calls) >= 6 * len(ADAM_SHAPES) + 2
+    for step in range(3, 6):
+        feed(ga, g_steps[step]); feed(gb, g_steps[step])
+        if step == 5:
+            prog_a.capture()
+        prog_a.run()
+        prog_b.run()
+        numpy_step(g_steps[step])
+        for i, (a, b) in enumerate(zip(pa, pb)):
+            exact(a.value.numpy(), b.value.numpy(), f"step {step} value {i}")
+            exact(opt_a.m_t[id(ga[i])].numpy(), opt_b.m_t[id(gb[i])].numpy(), f"step {step} first moment {i}")
+            exact(opt_a.v_t[id(ga[i])].numpy(), opt_b.v_t[id(gb[i])].numpy(), f"step {step} second moment {i}")
+        exact(opt_a.t.numpy(), opt_b.t.numpy(), "step counter")
+    prog_a.release_graph()
+    for i, a in enumerate(pa):
+        close(a.value.numpy(), w[i], 1e-4, f"value {i} vs float64")
+        close(opt_a.v_t[id(ga[i])].numpy(), v[i], 1e-5, f"second moment {i} vs float64")
+    close(opt_a.t.numpy(), np.array([t]), 1e-6, "step counter vs float64")
+    assert fused_launches <= 4
+
+    # the entry point validates everything before it launches
+    lib = ctx._lib
+    from sage_amd import abi
+    import ctypes as C
+    one = lambda x: (abi.sg_tensor * 1)(x.c())
+    hyper = abi.sg_adam_hyper(1e-2, 0.9, 0.999, 0.1, 0.001, 1e-8, 0.0)
+    step_t = opt_a.t.c()
+    small, big = pa[1].value, pa[2].value
+    before = small.numpy().copy()
+    with pytest.raises(abi.ShapeError):
+        ctx.check(lib.sg_adam_update(ctx.handle, 1, one(small), one(big), one(small), one(small), C.byref(step_t), C.byref(hyper)))
+    with pytest.raises(abi.ShapeError):  # step must be a single element
+        ctx.check(lib.sg_adam_update(ctx.handle, 1, one(small), one(small), one(small), one(small), C.byref(big.c()), C.byref(hyper)))
+    with pytest.raises(abi.DTypeError):
+        idx = S.Tensor.from_numpy(ctx, np.zeros(3, np.int32))
+        ctx.check(lib.sg_adam_update(ctx.handle, 1, one(small), one(idx), one(small), one(small), C.byref(step_t), C.byref(hyper)))
+    exact(small.numpy(), before, "failed calls change nothing")
+    assert lib.sg_adam_update(ctx.handle, 0, None, None, None, None, C.byref(step_t), C.byref(hyper)) == 0

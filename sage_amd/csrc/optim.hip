@@ -5,8 +5,8 @@
 // the other; replaying that as launches costs six per parameter (three kernels, three copies into the
 // persistent buffers): 252 launches of a few microseconds for the 42 parameters of ResNet-18, more
 // than the backward pass itself.  Here up to 32 parameters share a launch: a workgroup finds its
-// tensor in a table passed by value and every thread rewrites four consecutive elements of the two
-// moments and the value.
+// tensor in a table passed by value and every thread rewrites four pieces of four consecutive elements
+// of the two moments and the value (the two powers of beta, the costly part, are formed once per thread).
 //
 // The arithmetic is the reference's expression, operation for operation and without contraction
 // (this file is compiled with -ffp-contract=off, like the generated map kernels), so the result is
@@ -21,7 +21,7 @@
 namespace {
 
 constexpr int ADAM_MAX = 32;      // tensors per launch
-constexpr int ADAM_BLOCK = 1024;  // elements per workgroup: 256 threads x 4
+constexpr int ADAM_BLOCK = 4096;  // elements per workgroup: 256 threads x 4 pieces of 4
 
 struct AdamTensor {
     float *value;
@@ -56,28 +56,30 @@ __global__ void __launch_bounds__(256) adam_kernel(const AdamArgs a) {
     for (int i = 1; i < a.count; ++i)
         if (a.t[i].first_block <= blockIdx.x) k = i;
     const AdamTensor t = a.t[k];
-    const uint32_t i0 = (blockIdx.x - t.first_block) * ADAM_BLOCK + threadIdx.x * 4u;
-    if (i0 >= t.n) return;
+    const uint32_t base = (blockIdx.x - t.first_block) * ADAM_BLOCK + threadIdx.x * 4u;
+    if (base >= t.n) return;
     const float step = *a.step;
     const float den1 = -powf(a.beta1, step) + 1.0f, den2 = -powf(a.beta2, step) + 1.0f;
-    if (t.vec && i0 + 4 <= t.n) {
-        const f32x4 p4 = *reinterpret_cast<const f32x4 *>(t.value + i0), g4 = *reinterpret_cast<const f32x4 *>(t.grad + i0);
-        const f32x4 m4 = *reinterpret_cast<const f32x4 *>(t.m + i0), v4 = *reinterpret_cast<const f32x4 *>(t.v + i0);
-        float p[4] = {p4.x, p4.y, p4.z, p4.w}, m[4] = {m4.x, m4.y, m4.z, m4.w}, v[4] = {v4.x, v4.y, v4.z, v4.w};
-        const float g[4] = {g4.x, g4.y, g4.z, g4.w};
+    for (uint32_t i0 = base; i0 < t.n && i0 < base + ADAM_BLOCK; i0 += 1024u) {
+        if (t.vec && i0 + 4 <= t.n) {
+            const f32x4 p4 = *reinterpret_cast<const f32x4 *>(t.value + i0), g4 = *reinterpret_cast<const f32x4 *>(t.grad + i0);
+            const f32x4 m4 = *reinterpret_cast<const f32x4 *>(t.m + i0), v4 = *reinterpret_cast<const f32x4 *>(t.v + i0);
+            float p[4] = {p4.x, p4.y, p4.z, p4.w}, m[4] = {m4.x, m4.y, m4.z, m4.w}, v[4] = {v4.x, v4.y, v4.z, v4.w};
+            const float g[4] = {g4.x, g4.y, g4.z, g4.w};
 #pragma unroll
-        for (int j = 0; j < 4; ++j) adam_element(p[j], g[j], m[j], v[j], a, den1, den2);
-        *reinterpret_cast<f32x4 *>(t.m + i0) = f32x4{m[0], m[1], m[2], m[3]};
-        *reinterpret_cast<f32x4 *>(t.v + i0) = f32x4{v[0], v[1], v[2], v[3]};
-        *reinterpret_cast<f32x4 *>(t.value + i0) = f32x4{p[0], p[1], p[2], p[3]};
-    } else {
-        const uint32_t i1 = i0 + 4 < t.n ? i0 + 4 : t.n;
-        for (uint32_t i = i0; i < i1; ++i) {
-            float p = t.value[i], m = t.m[i], v = t.v[i];
-            adam_element(p, t.grad[i], m, v, a, den1, den2);
-            t.m[i] = m;
-            t.v[i] = v;
-            t.value[i] = p;
+            for (int j = 0; j < 4; ++j) adam_element(p[j], g[j], m[j], v[j], a, den1, den2);
+            *reinterpret_cast<f32x4 *>(t.m + i0) = f32x4{m[0], m[1], m[2], m[3]};
+            *reinterpret_cast<f32x4 *>(t.v + i0) = f32x4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<f32x4 *>(t.value + i0) = f32x4{p[0], p[1], p[2], p[3]};
+        } else {
+            const uint32_t i1 = i0 + 4 < t.n ? i0 + 4 : t.n;
+            for (uint32_t i = i0; i < i1; ++i) {
+                float p = t.value[i], m = t.m[i], v = t.v[i];
+                adam_element(p, t.grad[i], m, v, a, den1, den2);
+                t.m[i] = m;
+                t.v[i] = v;
+                t.value[i] = p;
+            }
         }
     }
 }

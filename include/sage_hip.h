@@ -241,11 +241,12 @@ int sg_gemm_batched(sg_ctx *ctx, int transpose_a, int transpose_b, const sg_tens
 int sg_matmul_strided(sg_ctx *ctx, const sg_tensor *a, const sg_tensor *b, const sg_tensor *c,
                       const sg_gemm_epilogue *epi);
 
-/* Name of the kernel instantiation a GEMM of this shape is dispatched to (tile sizes and operand
- * layouts are template arguments), as it appears in a rocprofv3 kernel trace.  The reference has one
- * fixed 8x8 kernel per transpose mode (gemm.rs:208-221); here the tile is chosen per shape. */
-int sg_gemm_kernel_name(sg_ctx *ctx, int64_t M, int64_t N, int64_t K, int64_t batch, int a_k_contiguous,
-                        int b_n_contiguous, char *buf, uint64_t cap);
+/* Name of the kernel instantiation the most recent product on this context launched (sg_gemm,
+ * sg_gemm_batched, sg_matmul_strided, sg_conv2d; for a split-K product: its first pass), as it appears
+ * in a rocprofv3 kernel trace: tile sizes, operand layouts, guarded loads and image addressing are
+ * template arguments.  The reference has one fixed 8x8 kernel per transpose mode (gemm.rs:208-221);
+ * here the instantiation is chosen per shape.  SG_ERR_ARG before the first product. */
+int sg_gemm_last_kernel_name(sg_ctx *ctx, char *buf, uint64_t cap);
 
 /* ---- convolution feeder: ops/conv.rs --------------------------------------------------------- */
 

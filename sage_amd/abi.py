@@ -90,7 +90,7 @@ PROTOTYPES = {
     "sg_gemm_noalloc": (C.c_int, [_CTX, C.c_int, C.c_int, _TP, _TP, _TP, C.POINTER(sg_gemm_epilogue)]),
     "sg_gemm_batched": (C.c_int, [_CTX, C.c_int, C.c_int, _TP, _TP, _TP, C.POINTER(sg_gemm_epilogue)]),
     "sg_matmul_strided": (C.c_int, [_CTX, _TP, _TP, _TP, C.POINTER(sg_gemm_epilogue)]),
-    "sg_gemm_kernel_name": (C.c_int, [_CTX, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_char_p, C.c_uint64]),
+    "sg_gemm_last_kernel_name": (C.c_int, [_CTX, C.c_char_p, C.c_uint64]),
     "sg_im2col": (C.c_int, [_CTX, _TP, _TP, _I32P, _I32P, _I32P, _I32P]),
     "sg_conv2d": (C.c_int, [_CTX, _TP, _TP, _TP, _I32P, _I32P, _I32P, C.POINTER(sg_gemm_epilogue)]),
     "sg_pool2d": (C.c_int, [_CTX, C.c_int, C.c_int, _TP, _TP, _I32P, _I32P, _I32P, _I32P]),

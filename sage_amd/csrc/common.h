@@ -49,6 +49,7 @@ struct sg_ctx {
     // stream capture (sg_graph_begin .. sg_graph_end): blocks allocated AND freed inside the captured
     // region are workspaces whose addresses are baked into the graph; they stay live with the graph
     bool capturing = false;
+    int last_gemm[7] = {0, 0, 0, 0, 0, 0, 0};  // template arguments of the most recent product kernel (BM 0: none yet)
     std::vector<void *> capture_allocs, capture_held;
     // errors
     std::string last_error;

@@ -681,7 +681,10 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *__restr
 template <int BM, int BN, int WAVES_M, bool GUARD>
 void launch_layouts(sg_ctx *ctx, const GemmP &p, dim3 grid, bool a_kc, bool b_nc) {
     dim3 block(NTHREADS);
-    if (p.conv.ohw) {  // image-addressed A (sg_conv2d): one instantiation per tile shape
+    const bool conv = p.conv.ohw != 0;
+    const int inst[7] = {BM, BN, WAVES_M, conv || a_kc, conv || b_nc, GUARD, conv};
+    for (int i = 0; i < 7; ++i) ctx->last_gemm[i] = inst[i];
+    if (conv) {  // image-addressed A (sg_conv2d): one instantiation per tile shape
         hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD, true>), grid, block, 0, ctx->stream, p);
         return;
     }
@@ -926,15 +929,12 @@ int check_f32(sg_ctx *ctx, const sg_tensor *a, const sg_tensor *b, const sg_tens
 
 }  // namespace
 
-extern "C" int sg_gemm_kernel_name(sg_ctx *ctx, int64_t M, int64_t N, int64_t K, int64_t batch, int a_k_contiguous,
-                                   int b_n_contiguous, char *buf, uint64_t cap) {
+extern "C" int sg_gemm_last_kernel_name(sg_ctx *ctx, char *buf, uint64_t cap) {
     if (!ctx || !buf || cap < 8) return SG_ERR_ARG;
-    const TileCfg &t = kTileCfgs[choose_tile(ctx->num_cus, (int)M, (int)N, (int)K, (int)batch)];
-    // the fast instantiation when the shape tiles exactly (operands assumed 16-byte aligned here)
-    const bool guard = M % t.bm != 0 || N % t.bn != 0 || K % (2 * BK) != 0;
-    // (the last argument is the image-addressed A operand of sg_conv2d)
-    snprintf(buf, cap, "gemm_mfma_kernel<%d, %d, %d, %s, %s, %s, false>", t.bm, t.bn, t.waves_m, a_k_contiguous ? "true" : "false",
-             b_n_contiguous ? "true" : "false", guard ? "true" : "false");
+    const int *t = ctx->last_gemm;
+    if (t[0] == 0) return sg_fail(ctx, SG_ERR_ARG, "sg_gemm_last_kernel_name: no product has been launched on this context");
+    snprintf(buf, cap, "gemm_mfma_kernel<%d, %d, %d, %s, %s, %s, %s>", t[0], t[1], t[2], t[3] ? "true" : "false", t[4] ? "true" : "false",
+             t[5] ? "true" : "false", t[6] ? "true" : "false");
     return SG_OK;
 }
 

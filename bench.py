@@ -216,6 +216,36 @@ def cpu_baseline_kind(entry):
     return entry
 
 
+LAYER_KEYS = ["wk", "bk", "wq", "bq", "wv", "bv", "wo", "bo", "ln1_g", "ln1_b", "w1", "b1", "w2", "b2", "ln2_g", "ln2_b"]
+
+
+def cpu_baseline_whole_model(bert, variant, layers, gpu_logits):
+    """The CPU oracle on the whole model the GPU leg timed: same weights, same token ids, embedding to
+    classifier (about 10 s at b32 x s128 on 16 threads).  The worst deviation of the GPU logits from the
+    oracle's is reported beside the rate."""
+    from oracle import oracle as O
+    ht = O.HT.from_numpy
+    it = iter(bert["arrays"])
+    exact = variant == "reference"
+    p = {"word_emb": ht(next(it)), "pos_emb": ht(next(it))}
+    if not exact:
+        p["seg_emb"] = ht(next(it))
+    p["emb_g"], p["emb_b"] = ht(next(it)), ht(next(it))
+    p["layers"] = [{k: ht(next(it)) for k in LAYER_KEYS} for _ in range(layers)]
+    p["wc"], p["bc"] = ht(next(it)), ht(next(it))
+    act, eps, cls = ("relu", 1e-5, 1) if exact else ("gelu", 1e-12, 0)
+    ids, seg = ht(bert["ids"].view(np.uint32)), None if bert["segment_ids"] is None else ht(bert["segment_ids"].view(np.uint32))
+    batch, seq = bert["ids"].shape
+    t0 = time.perf_counter()
+    lo = O.bert_forward(ids, ht(bert["mask"]), p, 12, act, eps, cls, seg)
+    dt = time.perf_counter() - t0
+    lo = lo.numpy().astype(np.float64)
+    dev = float(np.max(np.abs(gpu_logits - lo) / np.maximum(np.abs(lo), np.sqrt(np.mean(lo * lo)))))
+    return cpu_baseline_kind({"value": batch / dt, "unit": "seqs/s", "cores": O.num_threads(), "kind": "port",
+                              "sample": f"the whole {layers}-layer forward pass at b{batch} s{seq} (same weights and ids) in {dt:.1f} s",
+                              "gpu_vs_cpu_logits_worst_rel": dev})
+
+
 def cpu_baseline(variant, batch, seq, rng_seed):
     """The CPU oracle (oracle/: C restatement of the reference kernels, OpenMP over work-items) on one
     of the 12 encoder layers (whole batch at b32 x s128; at most 4096 tokens of it for larger shapes);
@@ -501,7 +531,8 @@ def main():
         model, arrays, x_host, logits = build_resnet18(ctx, batch, rng)
     else:
         batch = a.batch
-        cfg, model, logits = build_bert(ctx, a.variant, a.batch, a.seq, a.layers, rng)
+        bert = build_bert(ctx, a.variant, a.batch, a.seq, a.layers, rng, detail=True)
+        cfg, model, logits = bert["cfg"], bert["model"], bert["logits"]
     prog = S.Program(ctx, [logits])  # first evaluation: builds kernels, allocates every buffer
     ctx.sync()
     out0 = prog.outputs[0].numpy()
@@ -598,7 +629,12 @@ def main():
         ctx.trim()
         res["roofline_hbm"] = hbm_rooflines(ctx)
     if not a.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline_resnet18(model, arrays, x_host) if a.workload == "resnet18" else cpu_baseline(a.variant, a.batch, a.seq, 6)
+        if a.workload == "resnet18":
+            res["cpu_baseline"] = cpu_baseline_resnet18(model, arrays, x_host)
+        elif a.batch * a.seq <= 4096:
+            res["cpu_baseline"] = cpu_baseline_whole_model(bert, a.variant, a.layers, out0)
+        else:
+            res["cpu_baseline"] = cpu_baseline(a.variant, a.batch, a.seq, 6)
     print(json.dumps(res))
 
 

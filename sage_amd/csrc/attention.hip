@@ -43,6 +43,7 @@ struct AttnP {
     int64_t a_sb0, a_sb1;  // addend strides over the two batch axes (0 = broadcast); per key, stride 1
     float scale;
     int vec_q, vec_k, vec_v, vec_o;
+    int xcd_remap;  // workgroups of one (batch, head) on one XCD: they share its keys and values in that XCD's L2
 };
 
 // SPLIT = false: the four wavefronts take four groups of 32 queries and every wavefront walks all keys.
@@ -70,8 +71,17 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(SP
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ql = lane & 31, h = lane >> 5;
-    const int bt0 = blockIdx.y / p.nb1, bt1 = blockIdx.y % p.nb1;
-    const int q0 = blockIdx.x * QB + (SPLIT ? (wave & 1) : wave) * 32;
+    // Workgroup ids go round-robin over the 8 XCDs.  Remapped, XCD x takes the x-th eighth of the (pair, query tile)
+    // list, so the query tiles of one (batch, head) pair run on one XCD and fetch its keys and values into one L2.
+    unsigned bx = blockIdx.x, by = blockIdx.y;
+    if (p.xcd_remap) {
+        const unsigned id = by * gridDim.x + bx, per = gridDim.x * gridDim.y / 8u;
+        const unsigned nid = (id % 8u) * per + id / 8u;
+        by = nid / gridDim.x;
+        bx = nid % gridDim.x;
+    }
+    const int bt0 = by / p.nb1, bt1 = by % p.nb1;
+    const int q0 = bx * QB + (SPLIT ? (wave & 1) : wave) * 32;
     const int kw = SPLIT ? (wave >> 1) * 32 : 0;  // this wavefront's first key inside an LDS block
     const float *Q = p.q + bt0 * p.q_sb0 + bt1 * p.q_sb1;
     const float *K = p.k + bt0 * p.k_sb0 + bt1 * p.k_sb1;
@@ -346,6 +356,7 @@ extern "C" int sg_attention(sg_ctx *ctx, const sg_tensor *q, const sg_tensor *k,
     if (const char *e = getenv("SAGE_ATTENTION_SPLIT")) split = atoi(e) != 0;
     const int qb = split ? 64 : 128;
     dim3 grid((unsigned)((Lq + qb - 1) / qb), (unsigned)(nb0 * nb1));
+    p.xcd_remap = grid.x > 1 && (grid.x * grid.y) % 8 == 0;
     if (D == 64) {
         if (split) hipLaunchKernelGGL((attention_kernel<64, true>), grid, dim3(64 * NW), 0, ctx->stream, p);
         else hipLaunchKernelGGL((attention_kernel<64, false>), grid, dim3(64 * NW), 0, ctx->stream, p);

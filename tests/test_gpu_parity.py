@@ -725,6 +725,35 @@ def test_conv2d_abi_errors(ctx):
     ctx.sync()
 
 
+def test_last_product_kernel_name(ctx):
+    """sg_gemm_last_kernel_name names the instantiation the most recent product launched: tile, operand layouts,
+    guarded loads and image addressing, as a kernel trace prints it."""
+    say("last product kernel name")
+    lib = abi.lib()
+    arr = lambda a, b: (C.c_int32 * 2)(a, b)
+
+    def last():
+        buf = C.create_string_buffer(128)
+        ctx.check(lib.sg_gemm_last_kernel_name(ctx.handle, buf, 128))
+        return buf.value.decode()
+
+    rng = np.random.default_rng(3)
+    a, b = dev(ctx, rng.standard_normal((256, 64)).astype(np.float32)), dev(ctx, rng.standard_normal((64, 128)).astype(np.float32))
+    a.matmul(b).eval(ctx)
+    assert last() == "gemm_mfma_kernel<64, 64, 2, true, true, false, false>", last()
+    dev(ctx, rng.standard_normal((70, 33)).astype(np.float32)).matmul(dev(ctx, rng.standard_normal((33, 9)).astype(np.float32))).eval(ctx)
+    assert last().endswith("true, false>") and ", true, true, true, false>" in last(), last()   # guarded loads
+    for c, want in ((64, "gemm_mfma_kernel<64, 64, 2, true, true, false, true>"), (5, "true, true, true, true>")):
+        x = S.Tensor.from_numpy(ctx, rng.standard_normal((4, 8, 8, c)).astype(np.float32))
+        f = S.Tensor.from_numpy(ctx, rng.standard_normal((3, 3, c, 64)).astype(np.float32))
+        out = S.Tensor.uninit(ctx, [4, 8, 8, 64])
+        xc, fc, oc = x.c(), f.c(), out.c()
+        ctx.check(lib.sg_conv2d(ctx.handle, C.byref(xc), C.byref(fc), C.byref(oc), arr(1, 1), arr(1, 1), arr(1, 1), None))
+        assert last().endswith(want), last()   # image-addressed: unguarded with 16-channel slabs, guarded otherwise
+    assert lib.sg_gemm_last_kernel_name(ctx.handle, None, 128) == abi.ERR_ARG
+    ctx.sync()
+
+
 # ----------------------------------------------------------------------------- fused row operators
 @pytest.mark.parametrize("shape", [(64, 128), (5, 1000), (3, 4, 16, 16), (9, 1024), (2, 2052), (7, 10)])
 def test_softmax_fused_vs_composed_vs_oracle(ctx, shape):

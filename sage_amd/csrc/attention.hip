@@ -349,7 +349,7 @@ extern "C" int sg_attention(sg_ctx *ctx, const sg_tensor *q, const sg_tensor *k,
     if (nb0 * nb1 > 65535) return sg_fail(ctx, SG_ERR_SHAPE, "sg_attention: more than 65535 (batch x head) pairs");
     // Few workgroups of 128 queries (less than two per compute unit): halving the work units (see the kernel)
     // balances the SIMDs.  The split kernel is held to 168 registers so that three of its workgroups share a
-    // compute unit.  Measured at b32 x 12 heads (queries x keys): 23.1 against 25.0 us at 128 x 128, 37 against
+    // compute unit.  Measured at b32 x 12 heads (queries x keys): 23.0 against 25.0 us at 128 x 128 (22.3 with the XCD placement), 37 against
     // 43 at 128 x 256, 63.5 against 76 at 128 x 512, 15 against 22 at 64 x 128; slower once the chip is full anyway.
     const int64_t wgs128 = nb0 * nb1 * ((Lq + 127) / 128);
     bool split = wgs128 < 2 * (int64_t)(ctx->num_cus > 0 ? ctx->num_cus : 256);

@@ -897,6 +897,62 @@ def _merge_common_subgraphs(targets):
         canon[id(v)] = table.setdefault(key, v)
 
 
+def _is_relu_mask(m):
+    """m = float(x > 0), the factor of nn.rs:33-40; returns x or None."""
+    if m.value is not None or m.op != "unary" or m.attrs.get("name") != "cast_float":
+        return None
+    g = m.inputs[0]
+    if g.value is not None or g.op != "binary" or g.attrs.get("name") != "gt":
+        return None
+    z = g.inputs[1]
+    if z.value is None and z.op == "literal" and z.attrs.get("value") == 0.0 and z.dtype == FLOAT:
+        return g.inputs[0]
+    return None
+
+
+def _relu_masks_from_outputs(targets):
+    """Where y = float(x > 0) * x (relu, nn.rs:33-40) and the same factor float(x > 0) is also used elsewhere (the
+    backward pass multiplies the incoming gradient by it, map.rs:1014-1041), those other uses read float(y > 0)
+    instead: y > 0 exactly when x > 0 (y is x or 0; a NaN fails both tests), so no value changes, and x, left
+    with relu as its only consumer, can be folded into the product that makes it instead of being stored."""
+    order, seen, stack = [], set(), [(t, False) for t in targets]
+    while stack:
+        v, expanded = stack.pop()
+        if expanded:
+            order.append(v)
+            continue
+        if id(v) in seen:
+            continue
+        seen.add(id(v))
+        stack.append((v, True))
+        if v.value is None:
+            for i in v.inputs:
+                stack.append((i, False))
+    relu_of = {}  # id(mask node) -> (mask node, relu node)
+    for y in order:
+        if y.value is None and y.op == "binary" and y.attrs.get("name") == "mul":
+            for m, x in ((y.inputs[0], y.inputs[1]), (y.inputs[1], y.inputs[0])):
+                if _is_relu_mask(m) is x and id(m) not in relu_of:
+                    relu_of[id(m)] = (m, y)
+    if not relu_of:
+        return
+    from_output = {}
+    for v in order:
+        if v.value is not None or not any(id(i) in relu_of for i in v.inputs):
+            continue
+        new = []
+        for i in v.inputs:
+            hit = relu_of.get(id(i))
+            if hit is None or hit[1] is v:
+                new.append(i)
+                continue
+            y = hit[1]
+            if id(y) not in from_output:
+                from_output[id(y)] = binary_map(y, 0.0, "gt").float()
+            new.append(from_output[id(y)])
+        v.inputs = tuple(new)
+
+
 class _Evaluator:
     def __init__(self, ctx, targets, record=None):
         self.ctx = ctx
@@ -906,6 +962,7 @@ class _Evaluator:
         self.targets = {id(t) for t in targets}
         if _FUSION["on"]:
             _merge_common_subgraphs(targets)
+            _relu_masks_from_outputs(targets)
         # which shared nodes are stored once and which are recomputed in every consumer (session.rs:101-169)
         self.states = state_partition(targets, decide_only=True) if _FUSION["on"] else {}
         _allow_depth(targets)

@@ -393,3 +393,56 @@ def test_state_partition_follows_program_compile():
     ev = run(outs)
     assert id(u) in ev.computed and id(s_) in ev.computed          # materialised once
     assert id(w_) not in ev.computed and id(q) not in ev.computed  # fused into each consumer
+
+
+def test_relu_factor_is_read_from_the_output_outside_relu(monkeypatch):
+    """relu(h) = float(h > 0) * h (nn.rs:33-40); the backward pass multiplies by the same factor (map.rs:1014-1041).
+    Before evaluation every use of the factor outside relu itself is re-pointed at float(relu(h) > 0), which has the
+    same value for every h, so that h = x.W + b has one consumer and becomes the product's epilogue: one map launch
+    less, and the pre-activation is never stored."""
+    from sage_amd import nn
+    from sage_amd import var as V
+    from sage_amd.grad import grad
+
+    class Lib(_DryLib):
+        def __init__(self):
+            super().__init__()
+            self.log = []
+
+        def __getattr__(self, name):
+            def call(*a):
+                self.log.append(name)
+                return 0
+            return call
+
+    def build_and_run(ctx):
+        x, w, b = _data(ctx, 8, 16), _data(ctx, 16, 32), _data(ctx, 32)
+        h = x.matmul(w) + b
+        y = nn.relu(h)
+        loss = (y * y).sum([0, 1], False)
+        gw, gb = grad(loss, [w, b])
+        targets = [gw, gb, loss]
+        ev = V._Evaluator(ctx, targets)
+        for t in targets:
+            ev.get(t)
+        return h, y, ev
+
+    V.set_fusion(True)
+    ctx = _DryCtx()
+    ctx._lib = Lib()
+    h, y, ev = build_and_run(ctx)
+    mask = next(i for i in y.inputs if i is not h)
+    assert V._is_relu_mask(mask) is h
+    others = [v for v in ev.keep.values() if v is not y and any(i is mask for i in v.inputs)]
+    assert not others                                   # nothing but relu reads float(h > 0) any more
+    assert [u for u in ev.users[id(h)] if u.op != "binary" or u.attrs["name"] not in ("gt", "mul")] == []
+    assert id(h) not in ev.computed                     # folded into the product, never stored on its own
+    with_rewrite = ctx._lib.log.count("sg_map")
+
+    monkeypatch.setattr(V, "_relu_masks_from_outputs", lambda targets: None)
+    ctx2 = _DryCtx()
+    ctx2._lib = Lib()
+    h2, _, ev2 = build_and_run(ctx2)
+    assert id(h2) in ev2.computed                       # the reference's graph stores the pre-activation
+    assert ctx2._lib.log.count("sg_map") == with_rewrite + 1
+    assert ctx2._lib.log.count("sg_gemm") + ctx2._lib.log.count("sg_matmul_strided") == ctx._lib.log.count("sg_gemm") + ctx._lib.log.count("sg_matmul_strided")

@@ -44,6 +44,7 @@ struct AttnP {
     float scale;
     int vec_q, vec_k, vec_v, vec_o;
     int xcd_remap;  // workgroups of one (batch, head) on one XCD: they share its keys and values in that XCD's L2
+    sg_fastdiv d_gx, d_nb1;  // division by gridDim.x and by nb1 as a multiply-high
 };
 
 // SPLIT = false: the four wavefronts take four groups of 32 queries and every wavefront walks all keys.
@@ -54,7 +55,17 @@ struct AttnP {
 // may come to 1.5 per SIMD (b32, 12 heads, s128: 1536 units on 1024 SIMDs), i.e. two rounds with half
 // the chip idle in the second; split in two they are 3 per SIMD.  Three wavefronts per SIMD need the kernel
 // within 168 registers (the compiler is told so below; the unsplit kernel keeps 2, at 3 it would spill).
-template <int D, bool SPLIT>
+//
+// VEC = true: every operand row is 16-byte aligned, all global accesses are 16-byte ones and the code has no
+// scalar fallbacks.  A launch starts with a cold instruction cache, and what a workgroup executes before its
+// first MFMA is fetched line by line: at b32 x 12 heads x s128 the prologue (pointer arithmetic with two
+// integer divisions, eight guarded and doubly coded Q loads, the first K/V requests) took 6 of the kernel's
+// 22 us.  Hence: divisions by multiply-high, row indices clamped instead of guarded (a query past the end
+// computes on the last row and is not written; a key past the end reads the last row and is masked with
+// -inf), one code path per load.
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, sg_fastdiv d) { return (__umulhi(n, d.magic) + n) >> d.shift; }
+
+template <int D, bool SPLIT, bool VEC>
 __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(SPLIT ? 3 : 2, SPLIT ? 3 : 2))) attention_kernel(const AttnP p) {
     static_assert(D % 32 == 0 && D <= 64, "head size 32 or 64");
     constexpr int QB = SPLIT ? 64 : 32 * NW;   // queries per workgroup
@@ -77,10 +88,10 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(SP
     if (p.xcd_remap) {
         const unsigned id = by * gridDim.x + bx, per = gridDim.x * gridDim.y / 8u;
         const unsigned nid = (id % 8u) * per + id / 8u;
-        by = nid / gridDim.x;
-        bx = nid % gridDim.x;
+        by = fdiv(nid, p.d_gx);
+        bx = nid - by * gridDim.x;
     }
-    const int bt0 = by / p.nb1, bt1 = by % p.nb1;
+    const int bt0 = (int)fdiv(by, p.d_nb1), bt1 = (int)by - bt0 * p.nb1;
     const int q0 = bx * QB + (SPLIT ? (wave & 1) : wave) * 32;
     const int kw = SPLIT ? (wave >> 1) * 32 : 0;  // this wavefront's first key inside an LDS block
     const float *Q = p.q + bt0 * p.q_sb0 + bt1 * p.q_sb1;
@@ -88,21 +99,8 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(SP
     const float *V = p.v + bt0 * p.v_sb0 + bt1 * p.v_sb1;
     const float *A = p.add ? p.add + bt0 * p.a_sb0 + bt1 * p.a_sb1 : nullptr;
 
-    // Q^T operand of this lane: Q[q][8g + 4h + s] for g < NG, s < 4, pre-multiplied by nothing
+    // Q^T operand of this lane: Q[q][8g + 4h + s] for g < NG, s < 4 (filled below, through LDS)
     float qreg[NG][4];
-    {
-        const int q = q0 + ql;
-        const float *row = Q + (int64_t)q * p.q_sl;
-#pragma unroll
-        for (int g = 0; g < NG; ++g) {
-            f32x4 t = {0.f, 0.f, 0.f, 0.f};
-            if (q < p.Lq) {
-                if (p.vec_q) t = *reinterpret_cast<const f32x4 *>(row + 8 * g + 4 * h);
-                else { t.x = row[8 * g + 4 * h]; t.y = row[8 * g + 4 * h + 1]; t.z = row[8 * g + 4 * h + 2]; t.w = row[8 * g + 4 * h + 3]; }
-            }
-            qreg[g][0] = t.x; qreg[g][1] = t.y; qreg[g][2] = t.z; qreg[g][3] = t.w;
-        }
-    }
 
     floatx16 oacc[ND];
 #pragma unroll
@@ -119,15 +117,13 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(SP
         for (int i = 0; i < NLD; ++i) {
             const int f = tid + i * 64 * NW;
             const int row = f / ROWV, c = (f % ROWV) * 4;
-            const int key = kb0 + row;
-            f32x4 a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
-            if (key < p.Lk) {
-                const float *kp = K + (int64_t)key * p.k_sl + c, *vp = V + (int64_t)key * p.v_sl + c;
-                if (p.vec_k) a = *reinterpret_cast<const f32x4 *>(kp);
-                else { a.x = kp[0]; a.y = kp[1]; a.z = kp[2]; a.w = kp[3]; }
-                if (p.vec_v) b = *reinterpret_cast<const f32x4 *>(vp);
-                else { b.x = vp[0]; b.y = vp[1]; b.z = vp[2]; b.w = vp[3]; }
-            }
+            const int key = min(kb0 + row, p.Lk - 1);  // a key past the end repeats the last one (finite values); its mask is -inf
+            const float *kp = K + (int64_t)key * p.k_sl + c, *vp = V + (int64_t)key * p.v_sl + c;
+            f32x4 a, b;
+            if (VEC || p.vec_k) a = *reinterpret_cast<const f32x4 *>(kp);
+            else { a.x = kp[0]; a.y = kp[1]; a.z = kp[2]; a.w = kp[3]; }
+            if (VEC || p.vec_v) b = *reinterpret_cast<const f32x4 *>(vp);
+            else { b.x = vp[0]; b.y = vp[1]; b.z = vp[2]; b.w = vp[3]; }
             kreg[i] = a;
             vreg[i] = b;
         }
@@ -147,7 +143,38 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(SP
         if (tid < KB) lds_m[tid] = mreg;
     };
 
-    request(0);
+    // The workgroup's Q tile goes through LDS: fetched like K and V (16 lanes per 256-byte row, whole cache lines),
+    // then each lane picks its operand registers out of the tile.  Fetched straight into the operand layout, a load
+    // instruction touches 32 rows for 32 bytes each, and with twelve wavefronts per compute unit doing so at once
+    // the first-level cache's line rate, not memory, set the time (1.8 us of a 21 us kernel at b32 x 12 heads x s128).
+    {
+        constexpr int NQ = QB * ROWV / (64 * NW);
+        f32x4 qtmp[NQ];
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            const int f = tid + i * 64 * NW;
+            const int row = f / ROWV, c = (f % ROWV) * 4;
+            const int q = min((int)bx * QB + row, p.Lq - 1);  // a query past the end repeats the last one; it is not written
+            const float *src = Q + (int64_t)q * p.q_sl + c;
+            if (VEC || p.vec_q) qtmp[i] = *reinterpret_cast<const f32x4 *>(src);
+            else { qtmp[i].x = src[0]; qtmp[i].y = src[1]; qtmp[i].z = src[2]; qtmp[i].w = src[3]; }
+        }
+        request(0);  // the first K/V block is in flight behind the Q tile
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            const int f = tid + i * 64 * NW;
+            const int row = f / ROWV, c = (f % ROWV) * 4;
+            *reinterpret_cast<f32x4 *>(&(row < KB ? lds_k : lds_v)[(row % KB) * LD + c]) = qtmp[i];
+        }
+        __syncthreads();
+        const int mine = (SPLIT ? (wave & 1) : wave) * 32 + ql;
+        const float *src = &(mine < KB ? lds_k : lds_v)[(mine % KB) * LD + 4 * h];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            const f32x4 t = *reinterpret_cast<const f32x4 *>(src + 8 * g);
+            qreg[g][0] = t.x; qreg[g][1] = t.y; qreg[g][2] = t.z; qreg[g][3] = t.w;
+        }
+    }
     for (int kb0 = 0; kb0 < p.Lk; kb0 += KB) {
         __syncthreads();  // everyone is done reading the previous block
         deposit();
@@ -276,7 +303,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(SP
             float *dst = row + ND * (8 * g + 4 * h);
 #pragma unroll
             for (int c = 0; c < ND; ++c) {
-                if (p.vec_o) *reinterpret_cast<f32x4 *>(dst + 4 * c) = f32x4{t[4 * c], t[4 * c + 1], t[4 * c + 2], t[4 * c + 3]};
+                if (VEC || p.vec_o) *reinterpret_cast<f32x4 *>(dst + 4 * c) = f32x4{t[4 * c], t[4 * c + 1], t[4 * c + 2], t[4 * c + 3]};
                 else { dst[4 * c] = t[4 * c]; dst[4 * c + 1] = t[4 * c + 1]; dst[4 * c + 2] = t[4 * c + 2]; dst[4 * c + 3] = t[4 * c + 3]; }
             }
         }
@@ -357,13 +384,22 @@ extern "C" int sg_attention(sg_ctx *ctx, const sg_tensor *q, const sg_tensor *k,
     const int qb = split ? 64 : 128;
     dim3 grid((unsigned)((Lq + qb - 1) / qb), (unsigned)(nb0 * nb1));
     p.xcd_remap = grid.x > 1 && (grid.x * grid.y) % 8 == 0;
+    p.d_gx = sg_make_fastdiv(grid.x);
+    p.d_nb1 = sg_make_fastdiv((uint32_t)nb1);
+    const bool vec = p.vec_q && p.vec_k && p.vec_v && p.vec_o;
+#define SG_ATTN_LAUNCH(D_, SPLIT_)                                                                                             \
+    do {                                                                                                                       \
+        if (vec) hipLaunchKernelGGL((attention_kernel<D_, SPLIT_, true>), grid, dim3(64 * NW), 0, ctx->stream, p);            \
+        else hipLaunchKernelGGL((attention_kernel<D_, SPLIT_, false>), grid, dim3(64 * NW), 0, ctx->stream, p);               \
+    } while (0)
     if (D == 64) {
-        if (split) hipLaunchKernelGGL((attention_kernel<64, true>), grid, dim3(64 * NW), 0, ctx->stream, p);
-        else hipLaunchKernelGGL((attention_kernel<64, false>), grid, dim3(64 * NW), 0, ctx->stream, p);
+        if (split) SG_ATTN_LAUNCH(64, true);
+        else SG_ATTN_LAUNCH(64, false);
     } else {
-        if (split) hipLaunchKernelGGL((attention_kernel<32, true>), grid, dim3(64 * NW), 0, ctx->stream, p);
-        else hipLaunchKernelGGL((attention_kernel<32, false>), grid, dim3(64 * NW), 0, ctx->stream, p);
+        if (split) SG_ATTN_LAUNCH(32, true);
+        else SG_ATTN_LAUNCH(32, false);
     }
+#undef SG_ATTN_LAUNCH
     SG_CHECK_LAUNCH(ctx, "attention");
     return SG_OK;
 }

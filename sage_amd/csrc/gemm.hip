@@ -68,7 +68,7 @@ struct ConvG {
     int vec;                       // C % 4 == 0 and the image is 16-byte aligned: four channels per load
     int fast;                      // C % 16 == 0, at most 64 taps, the image below 2^31 bytes: a slab of 16 k is 16 channels
                                    // of ONE tap, so unguarded instantiations can fetch A with buffer loads (see the kernel)
-    int ntaps;                     // KH * KW
+    int KH;                        // kernel height
     uint32_t img_bytes;            // size of the whole image tensor (fast path only)
 };
 
@@ -354,11 +354,11 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
             const uint32_t oh = fdiv(r, p.conv.d_ow), ow = r - oh * (uint32_t)p.conv.OW;
             const int ih0 = (int)oh * p.conv.sh - p.conv.ph, iw0 = (int)ow * p.conv.sw - p.conv.pw;
             cf_off[i] = (uint32_t)(((n_img * (uint32_t)p.conv.H + (uint32_t)(ih0 + p.conv.ph)) * (uint32_t)p.conv.W + (uint32_t)(iw0 + p.conv.pw)) * (uint32_t)p.conv.C + (uint32_t)k) * 4u;
-            uint64_t mask = 0;
-            for (int t = 0; t < p.conv.ntaps; ++t) {
-                const int ky = t / p.conv.KW, kx = t - ky * p.conv.KW;
-                const int ih = ih0 + ky * p.conv.dh, iw = iw0 + kx * p.conv.dw;
-                if ((unsigned)ih < (unsigned)p.conv.H && (unsigned)iw < (unsigned)p.conv.W) mask |= 1ull << t;
+            uint64_t mask = 0, bit = 1;
+            for (int ky = 0, ih = ih0; ky < p.conv.KH; ++ky, ih += p.conv.dh) {
+                const bool row_inside = (unsigned)ih < (unsigned)p.conv.H;
+                for (int kx = 0, iw = iw0; kx < p.conv.KW; ++kx, iw += p.conv.dw, bit <<= 1)
+                    if (row_inside && (unsigned)iw < (unsigned)p.conv.W) mask |= bit;
             }
             cf_mask[i] = mask;
         }
@@ -1001,7 +1001,7 @@ extern "C" int sg_conv2d(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *filte
     g.d_c = sg_make_fastdiv((uint32_t)Cc); g.d_kw = sg_make_fastdiv((uint32_t)KW);
     const float *img = (const float *)x->base + x->offset;
     g.vec = Cc % 4 == 0 && ptr_aligned16(img);
-    g.ntaps = (int)(KH * KW);
+    g.KH = (int)KH;
     const int64_t img_bytes = N * H * W * Cc * 4, lead_bytes = ((int64_t)pad[1] * W + pad[0]) * Cc * 4;
     g.fast = Cc % 16 == 0 && ptr_aligned16(img) && KH * KW <= 64 && img_bytes + lead_bytes < (1ll << 31);
     g.img_bytes = g.fast ? (uint32_t)img_bytes : 0u;

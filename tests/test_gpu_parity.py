@@ -866,6 +866,40 @@ def test_attention_key_split_variant_matches(ctx, monkeypatch, split, n, h, lq, 
     close(out.numpy(), ref, REL_GEMM, "attention vs float64")
 
 
+@pytest.mark.parametrize("split", ["0", "1"])
+def test_attention_unaligned_operands(ctx, monkeypatch, split):
+    """Operands that are views at an odd element offset with a row stride of d + 1: no 16-byte access is legal,
+    the instantiation with scalar loads and stores runs; same result as float64 attention, and the padding
+    elements between the output rows stay untouched."""
+    say("attention on unaligned views, split", split)
+    monkeypatch.setenv("SAGE_ATTENTION_SPLIT", split)
+    lib = abi.lib()
+    from sage_amd.shape import Shape
+    n, h, lq, lk, d = 2, 3, 70, 100, 64
+    rng = np.random.default_rng(77)
+    ld = d + 1
+
+    def padded(l):
+        buf = rng.standard_normal(1 + n * h * l * ld).astype(np.float32)
+        view = buf[1:].reshape(n, h, l, ld)[..., :d]
+        return buf, view
+
+    (bq, q), (bk, k), (bv, v) = padded(lq), padded(lk), padded(lk)
+    bo = np.full(1 + n * h * lq * ld, 7.0, np.float32)
+    tensors = [S.Tensor.from_numpy(ctx, b) for b in (bq, bk, bv, bo)]
+    shapes = [Shape([n, h, l, d], [h * l * ld, l * ld, ld, 1], 1) for l in (lq, lk, lk, lq)]
+    qc, kc, vc, oc = (t.with_shape(sh).c() for t, sh in zip(tensors, shapes))
+    scale = 1.0 / np.sqrt(np.float32(d))
+    ctx.check(lib.sg_attention(ctx.handle, C.byref(qc), C.byref(kc), C.byref(vc), None, C.c_float(scale), C.byref(oc)))
+    s = np.einsum("nhqd,nhkd->nhqk", q.astype(np.float64), k.astype(np.float64)) * float(scale)
+    s -= np.maximum(s.max(-1, keepdims=True), 0.0)
+    p_ = np.exp(s)
+    ref = np.einsum("nhqk,nhkd->nhqd", p_ / p_.sum(-1, keepdims=True), v.astype(np.float64))
+    got = tensors[3].numpy()
+    close(got[1:].reshape(n, h, lq, ld)[..., :d], ref, REL_GEMM, "attention on unaligned views vs float64")
+    assert got[0] == 7.0 and np.all(got[1:].reshape(n, h, lq, ld)[..., d] == 7.0)
+
+
 def test_attention_fully_masked_row_is_reference_nan(ctx):
     """Every key masked by -1e5: the reference's softmax shifts by max(0, row max) = 0, every exp underflows
     and the row is 0/0.  The fused kernel keeps that behaviour instead of a uniform row."""

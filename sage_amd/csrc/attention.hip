@@ -54,7 +54,9 @@ struct AttnP {
 // large, which is what balances a short-sequence launch: B*H*L/32 units of 32 queries x all keys
 // may come to 1.5 per SIMD (b32, 12 heads, s128: 1536 units on 1024 SIMDs), i.e. two rounds with half
 // the chip idle in the second; split in two they are 3 per SIMD.  Three wavefronts per SIMD need the kernel
-// within 168 registers (the compiler is told so below; the unsplit kernel keeps 2, at 3 it would spill).
+// within 168 registers (the compiler is told so below).  The unsplit kernel with one code path per load fits
+// that limit too, but for three values spilled outside the key loop: a third workgroup per compute unit hides
+// the others' prologues (430 -> 417 us at b64 x 12 heads x s512); with scalar fallbacks it stays at two.
 //
 // VEC = true: every operand row is 16-byte aligned, all global accesses are 16-byte ones and the code has no
 // scalar fallbacks.  A launch starts with a cold instruction cache, and what a workgroup executes before its
@@ -66,7 +68,7 @@ struct AttnP {
 __device__ __forceinline__ uint32_t fdiv(uint32_t n, sg_fastdiv d) { return (__umulhi(n, d.magic) + n) >> d.shift; }
 
 template <int D, bool SPLIT, bool VEC>
-__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(SPLIT ? 3 : 2, SPLIT ? 3 : 2))) attention_kernel(const AttnP p) {
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((SPLIT || VEC) ? 3 : 2, (SPLIT || VEC) ? 3 : 2))) attention_kernel(const AttnP p) {
     static_assert(D % 32 == 0 && D <= 64, "head size 32 or 64");
     constexpr int QB = SPLIT ? 64 : 32 * NW;   // queries per workgroup
     constexpr int NKB = SPLIT ? 1 : KB / 32;   // 32-key MFMA blocks a wavefront takes from an LDS block

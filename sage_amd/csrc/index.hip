@@ -50,6 +50,20 @@ __global__ void __launch_bounds__(256) gather_kernel(const uint32_t *__restrict_
     y[gid] = x[xo + target * caxis_stride];
 }
 
+// Row gather: x [V, E] with unit inner stride, one index per output row (the index tensor is expanded along the
+// inner axis with stride 0, as Embedding::pass builds it, layers.rs:430-446): a thread copies 16 bytes of a row.
+// The general kernel above moves 4 bytes per thread behind a division per axis.
+__global__ void __launch_bounds__(256) gather_rows_kernel(const uint32_t *__restrict__ x, const uint32_t *__restrict__ ind,
+                                                          uint32_t *__restrict__ y, uint32_t n_vec, uint32_t vec_per_row, sg_fastdiv d_row,
+                                                          uint32_t x_row_stride, uint32_t ind_row_stride, uint32_t x_off, uint32_t ind_off) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
+    if (gid >= n_vec) return;
+    const uint32_t row = (__umulhi(gid, d_row.magic) + gid) >> d_row.shift, c = gid - row * vec_per_row;
+    const uint32_t target = ind[ind_off + row * ind_row_stride];
+    *reinterpret_cast<u32x4 *>(y + (size_t)gid * 4u) = *reinterpret_cast<const u32x4 *>(x + x_off + (size_t)target * x_row_stride + c * 4u);
+}
+
 template <class T>
 __global__ void __launch_bounds__(256) scatter_add_kernel(const T *__restrict__ x, const uint32_t *__restrict__ ind, T *__restrict__ y,
                                                           uint32_t n, Dims idims, Dims xdims, Dims ydims, int axis, uint32_t x_off,
@@ -224,6 +238,17 @@ extern "C" int sg_gather(sg_ctx *ctx, int axis, const sg_tensor *x, const sg_ten
         if (a != axis && ind->extents[a] > x->extents[a])
             return sg_fail(ctx, SG_ERR_SHAPE, "sg_gather: ind extent[%d] exceeds x's", a);
     const uint32_t n = (uint32_t)sg_numel(ind);
+    if (n == 0) return SG_OK;
+    if (x->rank == 2 && axis == 0 && ind->extents[1] > 1 && ind->strides[1] == 0 && x->strides[1] == 1 && ind->extents[1] % 4 == 0 &&
+        x->strides[0] % 4 == 0 && x->offset % 4 == 0 && (uintptr_t)x->base % 16 == 0 && ((uintptr_t)out->base + (uint64_t)out->offset * 4) % 16 == 0 &&
+        x->strides[0] >= 0 && ind->strides[0] >= 0 && x->strides[0] < (1ll << 31) && ind->strides[0] < (1ll << 31)) {
+        const uint32_t vec_per_row = (uint32_t)(ind->extents[1] / 4), n_vec = n / 4;
+        hipLaunchKernelGGL(gather_rows_kernel, dim3((n_vec + 255) / 256), dim3(256), 0, ctx->stream, (const uint32_t *)x->base,
+                           (const uint32_t *)ind->base, (uint32_t *)out->base + out->offset, n_vec, vec_per_row, sg_make_fastdiv(vec_per_row),
+                           (uint32_t)x->strides[0], (uint32_t)ind->strides[0], (uint32_t)x->offset, (uint32_t)ind->offset);
+        SG_CHECK_LAUNCH(ctx, "gather (rows)");
+        return SG_OK;
+    }
     Dims idims = dims_of(ind->extents, ind->strides, ind->rank), xdims = dims_of(x->extents, x->strides, x->rank);
     hipLaunchKernelGGL(gather_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, (const uint32_t *)x->base, (const uint32_t *)ind->base,
                        (uint32_t *)out->base + out->offset, n, idims, xdims, axis, (uint32_t)x->offset, (uint32_t)ind->offset);

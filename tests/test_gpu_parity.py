@@ -295,6 +295,14 @@ def test_gather_scatter(ctx):
     emb.weight.set(S.Tensor.from_numpy(ctx, w))
     exact(emb.pass_(dev(ctx, ids)).eval(ctx).numpy(), w[ids], "embedding")
     exact(O.embedding(ht(w), ht(ids)).numpy(), w[ids], "oracle embedding")
+    say("gather rows: 16-byte row path (wide table view, repeated ids) and its fallbacks (odd width, odd offset)")
+    big = rng.standard_normal((40, 24)).astype(np.float32)
+    ids2 = rng.integers(0, 40, (11,)).astype(np.uint32)
+    ids2[3] = ids2[7]
+    for lo, width in ((4, 16), (8, 12), (0, 24), (3, 16), (4, 10)):   # column window of the table: offset, width
+        table = dev(ctx, big).slice(1, lo, lo + width)
+        idx = dev(ctx, ids2).view([11, 1]).expand([11, width])
+        exact(table.gather(idx, 0).eval(ctx).numpy(), big[ids2, lo:lo + width], f"gather rows lo={lo} width={width}")
     say("gather from a transposed table")
     xd, xo = view_pair(ctx, x, lambda t: t.transpose(0, 2))
     ind = rng.integers(0, 7, (7, 6, 2)).astype(np.uint32)

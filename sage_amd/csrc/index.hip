@@ -182,11 +182,16 @@ __global__ void __launch_bounds__(256) im2col_kernel(const float *__restrict__ i
 // the additions run col_x outer, col_y inner, as the reference's, so the sum is bit-identical to a
 // sequential restatement.  The reference tests ker_x against dilation_h and ker_y against dilation_w
 // (conv.rs:463-465); kept, it only matters when the two dilations differ.
+// VEC = 4: a thread sums four consecutive channels (16-byte loads, one 16-byte store); each channel's additions
+// keep their order.
+template <int VEC>
 __global__ void __launch_bounds__(256) col2im_kernel(const float *__restrict__ col, float *__restrict__ img, uint32_t n_out, Im2colP p) {
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
     const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
     if (gid >= n_out) return;
-    const int c = gid % p.chan;
-    uint32_t t = gid / p.chan;
+    const uint32_t cv = p.chan / VEC;  // channel groups per pixel
+    const int c = (gid % cv) * VEC;
+    uint32_t t = gid / cv;
     const int img_x = t % p.img_w;
     t /= p.img_w;
     const int img_y = t % p.img_h;
@@ -198,17 +203,17 @@ __global__ void __launch_bounds__(256) col2im_kernel(const float *__restrict__ c
     const int col_x_end = min(img_x_pad / p.stride_w + 1, p.col_w);
     const int col_y_end = min(img_y_pad / p.stride_h + 1, p.col_h);
     const float *cb = col + (size_t)n * p.col_h * p.col_w * p.ker_h * p.ker_w * p.chan + c;
-    float val = 0.0f;
+    vec_t val = 0.0f;
     for (int col_x = col_x_start; col_x < col_x_end; ++col_x)
         for (int col_y = col_y_start; col_y < col_y_end; ++col_y) {
             int ker_x = img_x_pad - col_x * p.stride_w, ker_y = img_y_pad - col_y * p.stride_h;
             if (ker_x % p.dil_h == 0 && ker_y % p.dil_w == 0) {
                 ker_x /= p.dil_h;
                 ker_y /= p.dil_w;
-                val += cb[(size_t)(((col_y * p.col_w + col_x) * p.ker_h + ker_y) * p.ker_w + ker_x) * p.chan];
+                val += *reinterpret_cast<const vec_t *>(cb + (size_t)(((col_y * p.col_w + col_x) * p.ker_h + ker_y) * p.ker_w + ker_x) * p.chan);
             }
         }
-    img[gid] = val;
+    *reinterpret_cast<vec_t *>(img + (size_t)gid * VEC) = val;
 }
 
 }  // namespace
@@ -445,7 +450,10 @@ extern "C" int sg_col2im(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, 
     if (total >= (1ll << 32) || sg_numel(x) >= (1ll << 32)) return sg_fail(ctx, SG_ERR_SHAPE, "sg_col2im: more than 2^32 elements");
     const float *col = (const float *)x->base + x->offset;
     float *img = (float *)out->base + out->offset;
-    hipLaunchKernelGGL(col2im_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, col, img, (uint32_t)total, p);
+    if (p.chan % 4 == 0 && (uintptr_t)col % 16 == 0 && (uintptr_t)img % 16 == 0)
+        hipLaunchKernelGGL((col2im_kernel<4>), dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, ctx->stream, col, img, (uint32_t)(total / 4), p);
+    else
+        hipLaunchKernelGGL((col2im_kernel<1>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, col, img, (uint32_t)total, p);
     SG_CHECK_LAUNCH(ctx, "col2im");
     return SG_OK;
 }

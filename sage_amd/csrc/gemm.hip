@@ -724,7 +724,7 @@ int choose_split(int num_cus, int64_t wgs, int K, bool guarded_loop, int *k_chun
         if (wgs * 2 > cus) return 1;
         want = (int)(cus / wgs);
         if (want > K / 128) want = K / 128;
-        if (want > 32) want = 32;
+        if (want > 128) want = 128;
     }
     if (want < 2) return 1;
     int chunk = ((K + want - 1) / want + 31) / 32 * 32;

@@ -124,26 +124,36 @@ __global__ void __launch_bounds__(256) pool2d_kernel(const float *__restrict__ i
 #pragma unroll
     for (int e = 0; e < VEC; ++e) acc[e] = start;
     const float *base = img + (size_t)n * p.img_h * p.img_w * p.chan + c;
+    // up to four taps of a window column are requested before the first of them is combined (in tap order, so
+    // the result is that of the plain loop, which would wait for each tap in turn)
     for (int kx = 0; kx < p.ker_w; ++kx) {
         const int ix = (int)ox * p.stride_w - p.pad_w + kx * p.dil_w;
-        for (int ky = 0; ky < p.ker_h; ++ky) {
-            const int iy = (int)oy * p.stride_h - p.pad_h + ky * p.dil_h;
-            float v[VEC];
+        const bool col_inside = ix >= 0 && ix < p.img_w;
+        for (int ky0 = 0; ky0 < p.ker_h; ky0 += 4) {
+            float v[4][VEC];
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) v[e] = 0.0f;
-            if (ix >= 0 && ix < p.img_w && iy >= 0 && iy < p.img_h) {
-                const float *q = base + ((size_t)iy * p.img_w + ix) * p.chan;
-                if (VEC == 4) {
-                    const float4 t = *reinterpret_cast<const float4 *>(q);
-                    v[0] = t.x; v[1 % VEC] = t.y; v[2 % VEC] = t.z; v[3 % VEC] = t.w;
-                } else {
-                    v[0] = q[0];
+            for (int u = 0; u < 4; ++u) {
+                const int iy = (int)oy * p.stride_h - p.pad_h + (ky0 + u) * p.dil_h;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) v[u][e] = 0.0f;
+                if (ky0 + u < p.ker_h && col_inside && iy >= 0 && iy < p.img_h) {
+                    const float *q = base + ((size_t)iy * p.img_w + ix) * p.chan;
+                    if (VEC == 4) {
+                        const float4 t = *reinterpret_cast<const float4 *>(q);
+                        v[u][0] = t.x; v[u][1 % VEC] = t.y; v[u][2 % VEC] = t.z; v[u][3 % VEC] = t.w;
+                    } else {
+                        v[u][0] = q[0];
+                    }
                 }
             }
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                const float a = acc[e], b = v[e];
-                acc[e] = op == SG_R_SUM ? a + b : op == SG_R_PROD ? a * b : op == SG_R_MAX ? (a < b ? b : a) : (b < a ? b : a);
+            for (int u = 0; u < 4; ++u) {
+                if (ky0 + u >= p.ker_h) break;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float a = acc[e], b = v[u][e];
+                    acc[e] = op == SG_R_SUM ? a + b : op == SG_R_PROD ? a * b : op == SG_R_MAX ? (a < b ? b : a) : (b < a ? b : a);
+                }
             }
         }
     }

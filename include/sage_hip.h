@@ -289,8 +289,9 @@ int sg_rand_normal(sg_ctx *ctx, uint32_t seed_x, uint32_t seed_y, const sg_tenso
 
 /* ---- optimizer step: optim.rs ------------------------------------------------------------------ */
 
-/* Scalars of Adam (optim.rs:98-127).  one_minus_beta1/2 are passed, not derived: the reference forms
- * 1 - beta in f64 on the host and rounds once when the scalar enters the expression. */
+/* Scalars of Adam (optim.rs:98-127).  one_minus_beta1/2 are passed, not derived: the reference's
+ * beta1/beta2 are f32 fields and it forms `1.0 - self.beta` as an f32 subtraction on the host (optim.rs:152,
+ * 160): 1 - 0.9f = 0.100000024, 1 - 0.999f = 0.0009999871.  The caller passes those f32 differences. */
 typedef struct sg_adam_hyper {
     float lr, beta1, beta2, one_minus_beta1, one_minus_beta2, eps, weight_decay;
 } sg_adam_hyper;

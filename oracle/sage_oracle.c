@@ -15,7 +15,10 @@
  *   - every tensor literal the reference's own unit tests hold (tests/golden/reference_literals.json)
  *   - closed forms in float64 (numpy/scipy) for maps, reductions, GEMM, im2col (torch unfold);
  *     for col2im the adjoint identity <im2col(x), c> = <x, col2im(c)>
- *   - brute-force nested-loop index checks for translate_id / gather / scatter / slice windows.
+ *   - brute-force nested-loop index checks for translate_id / gather / scatter / slice windows and for the
+ *     batched product's four transpose modes;
+ *   - hand-worked known answers for the integer step and the scaling of the random fills, float64 math for
+ *     their Box-Muller transform.
  * Parity unpinned at ULP level: the reference evaluates exp/log/erf/pow/... and decides fma
  * contraction inside its vendor OpenCL driver, which is not part of the reference tree; these
  * restatements use the C library's float functions with contraction off.  The reference's own
@@ -701,14 +704,23 @@ int or_col2im(const sg_tensor *x, const sg_tensor *out, const int32_t ker[2], co
 }
 
 /* ---------------------------------------------------------------------------------------------
- * Uniform::compute / Normal::compute (rand.rs:39-49, 77-83, 120-136) for given seeds.  The odd
- * trailing element of the normal fill is the cosine branch only (the reference writes one float
- * past its buffer there).
+ * Uniform::compute / Normal::compute (rand.rs:39-49, 77-83, 120-136) for given seeds.
+ *
+ * The kernels are OpenCL C text built without compiler options (device.rs passes none), so an unsuffixed
+ * floating literal and M_PI are DOUBLE on the fp64-capable devices the reference selects:
+ *   xorshift128 returns (float)((double)rndint * 2.3283064e-10)   -- one rounding, not (float)rndint * 2^-32
+ *                                                                    (the two differ by an ulp for one seed in five);
+ *   theta = (float)(2 * M_PI * (double)u2);  rsq = -2 * log(u1) stays float (integer literal).
+ * The integer step is pinned by hand-worked known answers and the scaling by a seed on which the two readings
+ * differ (tests/test_oracle_golden.py); the Box-Muller values by float64 math.  log/cos/sin themselves are the C
+ * library's here and the driver's in the reference: unpinned at ULP level like every transcendental.
+ * The odd trailing element of the normal fill is the cosine branch only (the reference writes one float past
+ * its buffer there).
  * ------------------------------------------------------------------------------------------- */
 static float or_xorshift128(uint32_t seed_x, uint32_t seed_y) {
     const uint32_t t = seed_x ^ (seed_x << 11);
     const uint32_t rndint = seed_y ^ (seed_y >> 19) ^ (t ^ (t >> 8));
-    return (float)rndint * 2.3283064e-10f;
+    return (float)((double)rndint * 2.3283064e-10);
 }
 
 int or_rand_uniform(uint32_t seed_x, uint32_t seed_y, const sg_tensor *out) {
@@ -725,7 +737,7 @@ int or_rand_normal(uint32_t seed_x, uint32_t seed_y, const sg_tensor *out) {
         const float u1 = or_xorshift128(seed_x + (uint32_t)gid * 2u, seed_y);
         const float u2 = or_xorshift128(seed_x + (uint32_t)gid * 2u + 1u, seed_y);
         const float rsq = -2.0f * logf(u1);
-        const float theta = 2.0f * 3.14159265358979323846f * u2;
+        const float theta = (float)(2.0 * 3.14159265358979323846 * (double)u2);
         y[2 * gid] = sqrtf(rsq) * cosf(theta);
         if (2 * gid + 1 < n) y[2 * gid + 1] = sqrtf(rsq) * sinf(theta);
     }

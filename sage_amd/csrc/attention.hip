@@ -382,7 +382,7 @@ extern "C" int sg_attention(sg_ctx *ctx, const sg_tensor *q, const sg_tensor *k,
     // 43 at 128 x 256, 63.5 against 76 at 128 x 512, 15 against 22 at 64 x 128; slower once the chip is full anyway.
     const int64_t wgs128 = nb0 * nb1 * ((Lq + 127) / 128);
     bool split = wgs128 < 2 * (int64_t)(ctx->num_cus > 0 ? ctx->num_cus : 256);
-    if (const char *e = getenv("SAGE_ATTENTION_SPLIT")) split = atoi(e) != 0;
+    if (ctx->force_attention_split >= 0) split = ctx->force_attention_split != 0;  // measurement switch, fixed at context creation
     const int qb = split ? 64 : 128;
     dim3 grid((unsigned)((Lq + qb - 1) / qb), (unsigned)(nb0 * nb1));
     p.xcd_remap = grid.x > 1 && (grid.x * grid.y) % 8 == 0;

@@ -49,6 +49,11 @@ struct sg_ctx {
     // stream capture (sg_graph_begin .. sg_graph_end): blocks allocated AND freed inside the captured
     // region are workspaces whose addresses are baked into the graph; they stay live with the graph
     bool capturing = false;
+    // Measurement switches, read from the environment ONCE, when the context is created (so that two replays of
+    // one recorded program cannot round differently because the environment changed in between):
+    // SAGE_GEMM_SPLITK (1..128 k ranges, 0 = the heuristic), SAGE_GEMM_TILE (0..3, -1 = the heuristic),
+    // SAGE_ATTENTION_SPLIT (0/1, -1 = the heuristic).
+    int force_gemm_split = 0, force_gemm_tile = -1, force_attention_split = -1;
     int last_gemm[7] = {0, 0, 0, 0, 0, 0, 0};  // template arguments of the most recent product kernel (BM 0: none yet)
     std::vector<void *> capture_allocs, capture_held;
     // errors

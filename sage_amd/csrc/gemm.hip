@@ -37,6 +37,7 @@
 // order); the difference is fp32 rounding only and is covered by the 1e-3 GEMM tolerance.
 #include "common.h"
 
+#include <atomic>
 #include <type_traits>
 
 namespace {
@@ -56,7 +57,7 @@ constexpr int NUM_XCD = 8;
 constexpr int64_t SCRATCH_FLOATS = (int64_t)SG_GEMM_NOALLOC_SCRATCH_BYTES / 4;
 static __device__ __align__(256) float scratch[SCRATCH_FLOATS];
 constexpr int MAX_DEVICES = 64;
-float *g_scratch_ptr[MAX_DEVICES] = {};  // device address of `scratch` on each GPU, set by sg_gemm_device_setup
+std::atomic<float *> g_scratch_ptr[MAX_DEVICES];  // device address of `scratch` on each GPU (zero-initialised), set by sg_gemm_device_setup
 
 // Convolution as a GEMM whose A operand is never materialised: row m of A is output pixel
 // (n, oh, ow), column k is filter tap and channel (ky, kx, c), and A[m][k] is read from the image
@@ -710,12 +711,12 @@ bool needs_guard(const GemmP &p, int bm, int bn, bool a_kc, bool b_nc) {
 // How many k ranges to split into.  Splitting pays when the output has too few tiles to occupy the
 // chip and K is long: each range becomes its own workgroup (grid z) writing a partial product, and a
 // second kernel sums them.  Ranges are multiples of 32 so that the unguarded loop stays legal.
-int choose_split(int num_cus, int64_t wgs, int K, bool guarded_loop, int *k_chunk) {
-    const int64_t cus = num_cus > 0 ? num_cus : 256;
+int choose_split(const sg_ctx *ctx, int64_t wgs, int K, bool guarded_loop, int *k_chunk) {
+    const int64_t cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
     *k_chunk = 0;
-    const char *force = getenv("SAGE_GEMM_SPLITK");
+    const int force = ctx->force_gemm_split;  // a measurement switch, fixed when the context was created
     int want;
-    if (force) want = atoi(force);
+    if (force) want = force;
     else {
         // The matrix pipe of a compute unit is what a workgroup's loop occupies: two workgroups on one unit take
         // twice as long as one, so the ranges are cut so that tiles x ranges fills the units ONCE (measured on
@@ -746,7 +747,7 @@ int workspace(sg_ctx *ctx, int64_t floats, bool noalloc, void **ws) {
     if (floats > SCRATCH_FLOATS)
         return sg_fail(ctx, SG_ERR_ARG, "sg_gemm_noalloc: this product runs split-K and needs %lld bytes of workspace, "
                        "more than the %lld-byte static scratch (use sg_gemm)", (long long)floats * 4, (long long)SCRATCH_FLOATS * 4);
-    *ws = ctx->device >= 0 && ctx->device < MAX_DEVICES ? g_scratch_ptr[ctx->device] : nullptr;
+    *ws = ctx->device >= 0 && ctx->device < MAX_DEVICES ? g_scratch_ptr[ctx->device].load(std::memory_order_acquire) : nullptr;
     if (!*ws) return sg_fail(ctx, SG_ERR_DEVICE, "sg_gemm_noalloc: the static scratch of device %d was not set up", ctx->device);
     return SG_OK;
 }
@@ -769,7 +770,7 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noal
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     int k_chunk = 0;
-    const int nsplit = choose_split(ctx->num_cus, (int64_t)p.tiles_m * p.tiles_n * batch, p.K, needs_guard(p, BM, BN, a_kc, b_nc), &k_chunk);
+    const int nsplit = choose_split(ctx, (int64_t)p.tiles_m * p.tiles_n * batch, p.K, needs_guard(p, BM, BN, a_kc, b_nc), &k_chunk);
     if (nsplit > 1) {
         const int64_t slice = (int64_t)batch * p.M * p.N;
         void *ws = nullptr;
@@ -799,8 +800,9 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noal
 struct TileCfg { int bm, bn, waves_m; };
 const TileCfg kTileCfgs[] = {{128, 128, 2}, {128, 96, 4}, {128, 64, 2}, {64, 64, 2}};
 
-int choose_tile(int num_cus, int M, int N, int K, int batch) {
-    const int64_t cus = num_cus > 0 ? num_cus : 256;
+int choose_tile(const sg_ctx *ctx, int M, int N, int K, int batch) {
+    if (ctx->force_gemm_tile >= 0) return ctx->force_gemm_tile;
+    const int64_t cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
     int best = 3;
     double best_score = -1.0;
     for (int c = 0; c < 4; ++c) {
@@ -820,8 +822,6 @@ int choose_tile(int num_cus, int M, int N, int K, int batch) {
             best = c;
         }
     }
-    const char *force = getenv("SAGE_GEMM_TILE");
-    if (force && force[0] >= '0' && force[0] <= '3') best = force[0] - '0';
     return best;
 }
 
@@ -834,7 +834,7 @@ void launch_splitk_reduce(sg_ctx *ctx, const GemmP &p, const float *ws, int nspl
 }
 
 int launch_gemm(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noalloc) {
-    switch (choose_tile(ctx->num_cus, p.M, p.N, p.K, batch)) {
+    switch (choose_tile(ctx, p.M, p.N, p.K, batch)) {
     case 0: return launch_cfg<128, 128, 2>(ctx, p, batch, a_kc, b_nc, noalloc);
     case 1: return launch_cfg<128, 96, 4>(ctx, p, batch, a_kc, b_nc, noalloc);
     case 2: return launch_cfg<128, 64, 2>(ctx, p, batch, a_kc, b_nc, noalloc);
@@ -1003,7 +1003,13 @@ extern "C" int sg_conv2d(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *filte
     g.vec = Cc % 4 == 0 && ptr_aligned16(img);
     g.KH = (int)KH;
     const int64_t img_bytes = N * H * W * Cc * 4, lead_bytes = ((int64_t)pad[1] * W + pad[0]) * Cc * 4;
-    g.fast = Cc % 16 == 0 && ptr_aligned16(img) && KH * KW <= 64 && img_bytes + lead_bytes < (1ll << 31);
+    // The unguarded loads send an outside tap to lane offset 2^31 and rely on the descriptor's range check, which
+    // compares against (range - scalar offset): that difference must not wrap, so the largest scalar offset of
+    // the loop (last tap's displacement + the last 16-channel slab, + the 64 bytes it reads) has to lie inside
+    // the range; a dilation or padding larger than the image (N = 1) can exceed it and takes the guarded loads.
+    const int64_t max_slab_off = (((KH - 1) * (int64_t)dil[1] * W + (KW - 1) * (int64_t)dil[0]) * Cc + (Cc >= 16 ? Cc - 16 : 0)) * 4 + 64;
+    g.fast = Cc % 16 == 0 && ptr_aligned16(img) && KH * KW <= 64 && img_bytes + lead_bytes < (1ll << 31) &&
+             max_slab_off <= img_bytes + lead_bytes;
     g.img_bytes = g.fast ? (uint32_t)img_bytes : 0u;
     // A = the virtual [M, K] column matrix (row stride K, never dereferenced through it), B = filter as [K, OC], C = out as [M, OC]
     Mat ma{img, 0, 0, K, 1};
@@ -1016,10 +1022,11 @@ extern "C" int sg_conv2d(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *filte
 // on that GPU once (each GPU holds its own copy of the array at its own address).
 int sg_gemm_device_setup(sg_ctx *ctx) {
     if (ctx->device < 0 || ctx->device >= MAX_DEVICES) return SG_OK;  // sg_gemm_noalloc reports it when used
-    if (g_scratch_ptr[ctx->device]) return SG_OK;
+    if (g_scratch_ptr[ctx->device].load(std::memory_order_acquire)) return SG_OK;
     float *ptr = nullptr;
     SG_HIP(ctx, hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
-    g_scratch_ptr[ctx->device] = ptr;
+    // contexts created at the same time on several threads all resolve the same address: whichever store lands is right
+    g_scratch_ptr[ctx->device].store(ptr, std::memory_order_release);
     return SG_OK;
 }
 

@@ -9,11 +9,13 @@
 
 namespace {
 
-// rand.rs:39-49
+// rand.rs:39-49.  The reference's kernel text is OpenCL C built without options, where the unsuffixed literal is a
+// double: the product is formed in double and rounded to float once (one seed in five gives a different last
+// bit than (float)rndint * 2^-32 would).
 __device__ __forceinline__ float xorshift128(uint32_t seed_x, uint32_t seed_y) {
     const uint32_t t = seed_x ^ (seed_x << 11);
     const uint32_t rndint = seed_y ^ (seed_y >> 19) ^ (t ^ (t >> 8));
-    return (float)rndint * 2.3283064e-10f;
+    return (float)((double)rndint * 2.3283064e-10);
 }
 
 // rand.rs:77-83: y[gid] = xorshift128(seed_x + gid, seed_y + gid)
@@ -30,7 +32,7 @@ __global__ void __launch_bounds__(256) rand_normal_kernel(float *__restrict__ y,
     const float u1 = xorshift128(seed_x + gid * 2u, seed_y);
     const float u2 = xorshift128(seed_x + gid * 2u + 1u, seed_y);
     const float rsq = -2.0f * logf(u1);
-    const float theta = 2.0f * 3.14159265358979323846f * u2;
+    const float theta = (float)(2.0 * 3.14159265358979323846 * (double)u2);  // `2 * M_PI * u2`: M_PI is a double in OpenCL C
     const float r = sqrtf(rsq);
     y[2u * gid] = r * cosf(theta);
     if (2u * gid + 1u < n) y[2u * gid + 1u] = r * sinf(theta);

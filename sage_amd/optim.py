@@ -23,6 +23,13 @@ from .tensor import Tensor
 from .var import Var, evaluate, params_changed, scalar
 
 
+def _one_minus(x):
+    """1 - x as the reference forms it: its hyper-parameters are f32 fields and `1.0 - self.beta1` is an f32
+    subtraction (optim.rs:152, 160; 1 - 0.999f = 0.0009999871, not 0.001f)."""
+    import numpy as np
+    return float(np.float32(1.0) - np.float32(x))
+
+
 def _value(grad, ctx):
     if grad.value is None:
         evaluate(ctx, [grad])
@@ -91,7 +98,7 @@ class Sgd(Optimizer):
             g = gv + param * self.weight_decay if self.weight_decay != 0.0 else gv
             if self.momentum != 0.0:
                 if id(grad) not in self.b:
-                    b = Var.new(self.b[id(grad)]) * self.momentum + g * (1.0 - self.dampening)  # optim.rs:67-69
+                    b = Var.new(self.b[id(grad)]) * self.momentum + g * _one_minus(self.dampening)  # optim.rs:67-69
                 else:
                     b = g
                 self.b[id(grad)] = b.eval(ctx)
@@ -138,13 +145,13 @@ class Adam(Optimizer):
             g = gv + param * self.weight_decay if self.weight_decay != 0.0 else gv
             key = id(grad)
             if key in self.m_t:
-                m_t = Var.new(self.m_t[key]) * self.beta1 + g * (1.0 - self.beta1)
+                m_t = Var.new(self.m_t[key]) * self.beta1 + g * _one_minus(self.beta1)
             else:
                 m_t = scalar(0.0, grad.extents)
             self.m_t[key] = m_t.eval(ctx)
             m_t = Var.new(self.m_t[key])
             if key in self.v_t:
-                v_t = Var.new(self.v_t[key]) * self.beta2 + g.pow(2.0) * (1.0 - self.beta2)
+                v_t = Var.new(self.v_t[key]) * self.beta2 + g.pow(2.0) * _one_minus(self.beta2)
             else:
                 v_t = scalar(0.0, grad.extents)
             self.v_t[key] = v_t.eval(ctx)
@@ -169,8 +176,8 @@ class Adam(Optimizer):
             gv = Var.new(_value(grad, ctx))
             g = gv + param * self.weight_decay if self.weight_decay != 0.0 else gv
             key = id(grad)
-            m_t = Var.new(self.m_t[key]) * self.beta1 + g * (1.0 - self.beta1)
-            v_t = Var.new(self.v_t[key]) * self.beta2 + g.pow(2.0) * (1.0 - self.beta2)
+            m_t = Var.new(self.m_t[key]) * self.beta1 + g * _one_minus(self.beta1)
+            v_t = Var.new(self.v_t[key]) * self.beta2 + g.pow(2.0) * _one_minus(self.beta2)
             m_hat = m_t / (-scalar(self.beta1, [1]).pow(t) + 1.0)
             v_hat = v_t / (-scalar(self.beta2, [1]).pow(t) + 1.0)
             pairs += [(m_t, self.m_t[key]), (v_t, self.v_t[key]),
@@ -195,7 +202,7 @@ class Adam(Optimizer):
             for col, x in zip(cols, (param.value, grad.value, self.m_t[id(grad)], self.v_t[id(grad)])):
                 col.append(x)
         arrays = [(abi.sg_tensor * max(n, 1))(*[x.c() for x in col]) for col in cols]
-        hyper = abi.sg_adam_hyper(self.lr, self.beta1, self.beta2, 1.0 - self.beta1, 1.0 - self.beta2, self.eps, self.weight_decay)
+        hyper = abi.sg_adam_hyper(self.lr, self.beta1, self.beta2, _one_minus(self.beta1), _one_minus(self.beta2), self.eps, self.weight_decay)
         step = self.t.c()
         prog = _compile(ctx, [])
         args = (C.c_int(n), *arrays, C.byref(step), C.byref(hyper))

@@ -1197,7 +1197,7 @@ class _Evaluator:
     # ---- reductions and indexing
     def _ev_reduce(self, v):
         col = v.inputs[0]
-        if (_FUSION["on"] and col.op == "im2col" and self._private(col) and sorted(v.attrs["axes"]) == [3, 4]
+        if (_FUSION["on"] and col.op == "im2col" and self._private(col) and list(v.attrs["axes"]) == [3, 4]  # ky innermost, the kernel's order
                 and v.dtype == FLOAT and os.environ.get("SAGE_FUSE_CONV", "1") != "0"):
             # max_pool_2d / avg_pool_2d (conv.rs:143-165): the window is reduced while it is read, no column tensor
             x = self.get(col.inputs[0])
@@ -1365,6 +1365,10 @@ class _Evaluator:
         a = col.attrs
         n, oh, ow, kh, kw, c = col.extents
         if f.rank != 4 or f.extents[:3] != [kh, kw, c] or a["ker"] != [kw, kh]:
+            return None
+        # the product must be exactly [n*oh*ow, kh*kw*c] . [kh*kw*c, oc]: any other 2-D factorisation of the column
+        # tensor or of the filter is a different contraction and runs as im2col + gemm
+        if list(g.inputs[0].extents) != [n * oh * ow, kh * kw * c] or list(g.inputs[1].extents) != [kh * kw * c, f.extents[3]]:
             return None
         x, ft = self.get(col.inputs[0]), self.get(f)
         if not x.is_dense():

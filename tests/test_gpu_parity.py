@@ -25,6 +25,22 @@ def ctx():
     c.close()
 
 
+@pytest.fixture
+def ctx_under(monkeypatch):
+    """ctx_under(NAME=value, ..) -> a context created AFTER those environment switches were set: the library reads its
+    measurement switches once, when a context is created."""
+    made = []
+
+    def make(**env):
+        for k, v in env.items():
+            monkeypatch.setenv(k, v)
+        made.append(S.Context())
+        return made[-1]
+    yield make
+    for c in made:
+        c.close()
+
+
 @pytest.fixture(autouse=True)
 def _fusion_on():
     V.set_fusion(True)
@@ -352,13 +368,13 @@ def test_gemm_modes(ctx, mkn, ta, tb):
 @pytest.mark.parametrize("mkn,split", [((128, 4608, 512), None), ((512, 2304, 256), None), ((64, 1024, 64), None),
                                        ((70, 999, 33), "5"), ((130, 257, 70), "3"), ((128, 512, 128), "32"), ((37, 2000, 41), "7")])
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
-def test_gemm_split_k(ctx, monkeypatch, mkn, split, ta, tb):
+def test_gemm_split_k(ctx, ctx_under, mkn, split, ta, tb):
     """Few output tiles and a long K: the k range is split over workgroups and summed by a second kernel
     (chosen by itself for the first three shapes, forced for the ragged ones), with the epilogue behind it."""
     m, k, n = mkn
     say("gemm split-K", mkn, split, ta, tb)
     if split:
-        monkeypatch.setenv("SAGE_GEMM_SPLITK", split)
+        ctx = ctx_under(SAGE_GEMM_SPLITK=split)
     rng = np.random.default_rng(m + k + n)
     a = rng.uniform(-1, 1, (k, m) if ta else (m, k)).astype(np.float32)
     b = rng.uniform(-1, 1, (n, k) if tb else (k, n)).astype(np.float32)
@@ -430,9 +446,9 @@ def test_gemm_random_shapes_and_layouts(ctx):
         close(out, yo.numpy(), REL_GEMM, f"case {case} vs oracle")
 
 
-def test_gemm_batched_split_k(ctx, monkeypatch):
+def test_gemm_batched_split_k(ctx_under):
     say("gemm_batched split-K")
-    monkeypatch.setenv("SAGE_GEMM_SPLITK", "4")
+    ctx = ctx_under(SAGE_GEMM_SPLITK="4")
     rng = np.random.default_rng(77)
     bt, m, k, n = 3, 37, 300, 44
     a = rng.uniform(-1, 1, (bt, m, k)).astype(np.float32)
@@ -443,12 +459,12 @@ def test_gemm_batched_split_k(ctx, monkeypatch):
 
 
 @pytest.mark.parametrize("split", [None, "3"])
-def test_matmul_strided_residual_with_flattened_batch(ctx, monkeypatch, split):
+def test_matmul_strided_residual_with_flattened_batch(ctx, ctx_under, split):
     """C has two batch axes [2,3,M,N]; the residual is [6,M,N] (batch axes flattened), [2,3,M,N] or a
     single [M,N]-per-batch view: all three address batch entry b0*3+b1 (straight through the C ABI)."""
     say("matmul_strided residual layouts", split)
     if split:
-        monkeypatch.setenv("SAGE_GEMM_SPLITK", split)
+        ctx = ctx_under(SAGE_GEMM_SPLITK=split)
     lib = abi.lib()
     rng = np.random.default_rng(91)
     b0, b1, m, k, n = 2, 3, 40, 96, 36
@@ -648,6 +664,9 @@ CONV_CASES = [
     (8, 4, 4, 128, 1, 1, 64, [2, 2], [0, 0], [1, 1]),     # 1x1 stride 2 downsample: M = 32 ... guarded; and
     (32, 4, 4, 128, 1, 1, 64, [2, 2], [0, 0], [1, 1]),    # the same at M = 128: unguarded
     (64, 2, 2, 256, 3, 3, 256, [1, 1], [1, 1], [1, 1]),   # M = 256, K = 2304: unguarded and split-K
+    # dilation and padding larger than the image, one image: exactly tiled (M = 64, K = 288, C % 16 == 0), but the last taps'
+    # displacement lies beyond the image plus its lead, so the host must choose the guarded loads
+    (1, 8, 8, 32, 3, 3, 64, [1, 1], [9, 9], [9, 9]),
 ]
 
 
@@ -688,6 +707,26 @@ def test_conv2d_without_column_matrix(ctx, monkeypatch, case):
         else:
             exact(y_fused, y_explicit, "conv2d vs im2col + gemm")
         assert fused_launches <= (2 if with_epilogue else 1), fused_launches
+
+
+def test_product_over_another_factorisation_of_the_column_tensor_is_not_a_convolution(ctx):
+    """A product whose operands are OTHER 2-D views of an im2col tensor and of a rank-4 [kh,kw,c,*] filter is a
+    different contraction than conv_2d: it must run as im2col + gemm (two launches), not be handed to sg_conv2d."""
+    say("gemm over a re-factored column tensor")
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((1, 4, 4, 2)).astype(np.float32)
+    f = rng.standard_normal((2, 2, 2, 6)).astype(np.float32)
+    col = V.im2col(dev(ctx, x), 2, 1, 0, 1)                      # [1,3,3,2,2,2] = 72 elements
+    n0 = ctx.launches
+    y = V.gemm(col.reshape([18, 4]), dev(ctx, f).reshape([4, 12]), False, False).eval(ctx).numpy()
+    assert ctx.launches - n0 == 2
+    colo = O.im2col(ht(x), [2, 2], [1, 1], [0, 0], [1, 1]).numpy().reshape(18, 4)
+    close(y, colo.astype(np.float64) @ f.reshape(4, 12).astype(np.float64), REL_GEMM, "re-factored product")
+    # the true convolution over the same operands is one launch
+    n0 = ctx.launches
+    yc = V.conv_2d(dev(ctx, x), dev(ctx, f), 1, 0, 1).eval(ctx).numpy()
+    assert ctx.launches - n0 == 1
+    close(yc.reshape(9, 6), O.im2col(ht(x), [2, 2], [1, 1], [0, 0], [1, 1]).numpy().reshape(9, 8).astype(np.float64) @ f.reshape(8, 6).astype(np.float64), REL_GEMM, "conv_2d")
 
 
 @pytest.mark.parametrize("geom", [((2, 12, 10, 8), 3, 2, 1, 1), ((3, 14, 14, 64), 3, 2, 1, 1), ((2, 9, 7, 5), [2, 3], [1, 2], [1, 0], [2, 1]),
@@ -849,12 +888,12 @@ def test_attention_fused_vs_composed_vs_oracle(ctx, n, h, lq, lk, d, masked):
 
 @pytest.mark.parametrize("split", ["0", "1"])
 @pytest.mark.parametrize("n,h,lq,lk,d", [(2, 3, 128, 128, 64), (1, 2, 70, 200, 64), (2, 2, 33, 31, 32), (1, 1, 64, 300, 64)])
-def test_attention_key_split_variant_matches(ctx, monkeypatch, split, n, h, lq, lk, d):
+def test_attention_key_split_variant_matches(ctx_under, split, n, h, lq, lk, d):
     """The kernel that gives the two 32-key halves of every key block to different wavefronts and merges their
     online-softmax states, forced on and off: both agree with float64 attention (ragged key counts leave one half
     partly or wholly past the end)."""
     say("attention key split", split, (n, h, lq, lk, d))
-    monkeypatch.setenv("SAGE_ATTENTION_SPLIT", split)
+    ctx = ctx_under(SAGE_ATTENTION_SPLIT=split)
     lib = abi.lib()
     rng = np.random.default_rng(lq * 7 + lk)
     q, k, v = (rng.standard_normal((n, h, l, d)).astype(np.float32) for l in (lq, lk, lk))
@@ -875,12 +914,12 @@ def test_attention_key_split_variant_matches(ctx, monkeypatch, split, n, h, lq, 
 
 
 @pytest.mark.parametrize("split", ["0", "1"])
-def test_attention_unaligned_operands(ctx, monkeypatch, split):
+def test_attention_unaligned_operands(ctx_under, split):
     """Operands that are views at an odd element offset with a row stride of d + 1: no 16-byte access is legal,
     the instantiation with scalar loads and stores runs; same result as float64 attention, and the padding
     elements between the output rows stay untouched."""
     say("attention on unaligned views, split", split)
-    monkeypatch.setenv("SAGE_ATTENTION_SPLIT", split)
+    ctx = ctx_under(SAGE_ATTENTION_SPLIT=split)
     lib = abi.lib()
     from sage_amd.shape import Shape
     n, h, lq, lk, d = 2, 3, 70, 100, 64

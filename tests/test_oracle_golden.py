@@ -206,3 +206,105 @@ def test_embedding(golden):
     idx = golden("src/layers.rs", "test_embedding", "idx", np.int32)
     y = O.embedding(T(w), T(idx).view([4, 1]))
     assert np.array_equal(y.numpy().reshape(4, 24), w[:4])
+
+
+# ---- pins for what the reference holds no vector for ---------------------------------------------------------
+
+
+def test_xorshift128_known_answers():
+    """rand.rs:39-48 worked by hand (32-bit registers; `<<` drops the bits shifted out, `>>` is logical):
+
+        t = x ^ (x << 11);  rndint = y ^ (y >> 19) ^ (t ^ (t >> 8));  return rndint * 2.3283064e-10  [double literal]
+
+    (1, 2):                   t = 0x801,       t ^ (t>>8) = 0x801 ^ 0x8 = 0x809;          y ^ (y>>19) = 2            -> 0x80b = 2059
+    (0x80000001, 0xC0000000): x<<11 = 0x800 (bit 31 falls off), t = 0x80000801, t>>8 = 0x00800008 (no sign fill),
+                              t ^ (t>>8) = 0x80800809;  y>>19 = 0x1800, y ^ (y>>19) = 0xC0001800               -> 0x40801009
+    (0xFFFFFFFF, 0xFFFFFFFF): x<<11 = 0xFFFFF800, t = 0x7FF, t ^ (t>>8) = 0x7FF ^ 0x7 = 0x7F8;  y ^ (y>>19) = 0xFFFFFFFF ^ 0x1FFF
+                              = 0xFFFFE000                                                                    -> 0xFFFFE7F8
+    The uniform fill evaluates element gid at (seed_x + gid, seed_y + gid) (rand.rs:77-83), so element 0 of a fill
+    seeded with the pair is the pair's value.  The last case is a seed on which rounding the double product once
+    differs from (float)rndint * 2^-32: rndint = 0x98C4D688, product 0.59675350035.. -> 0x3F18C4D6 (the float-only
+    form gives 0x3F18C4D7)."""
+    cases = [((1, 2), 2059, 0x3500B000), ((0x80000001, 0xC0000000), 0x40801009, 0x3E810020),
+             ((0xFFFFFFFF, 0xFFFFFFFF), 0xFFFFE7F8, 0x3F7FFFE8), ((0x16, 0x98C47536), 0x98C4D688, 0x3F18C4D6)]
+    for (sx, sy), rndint, bits in cases:
+        u = O.rand_uniform([1], sx, sy).numpy()
+        assert u.view(np.uint32)[0] == bits, (hex(sx), hex(sy), hex(int(u.view(np.uint32)[0])))
+        # the stored bits are the float nearest to rndint * 2.3283064e-10 (one rounding of the double product)
+        assert np.float32(rndint * 2.3283064e-10).view(np.uint32) == bits
+    # element gid of a fill uses (seed_x + gid, seed_y + gid), wrapping at 2^32: elements 1 and 2 of a fill seeded
+    # (0xFFFFFFFF, 0) are the values of (0, 1) and (1, 2); (0, 1): t = 0, rndint = 1
+    u = O.rand_uniform([3], 0xFFFFFFFF, 0).numpy().view(np.uint32)
+    assert u[1] == np.float32(1 * 2.3283064e-10).view(np.uint32) and u[2] == 0x3500B000
+
+
+def test_box_muller_against_float64():
+    """rand.rs:120-136: pair p of a normal fill is sqrt(-2 ln u1) * (cos, sin)(2 pi u2) with u1, u2 the uniform values
+    of (seed_x + 2p, seed_y) and (seed_x + 2p + 1, seed_y) -- seed_y is NOT advanced, unlike the uniform fill; an odd
+    element count keeps the last cosine only.  Uniform values come from the integer step restated here with Python
+    integers (pinned above), the transform from float64 `math`."""
+    import math
+
+    def u(x, y):
+        x &= 0xFFFFFFFF
+        t = (x ^ (x << 11)) & 0xFFFFFFFF
+        return float(np.float32(((y ^ (y >> 19)) ^ (t ^ (t >> 8))) * 2.3283064e-10))
+
+    sx, sy, n = 0x9E3779B9, 0x7F4A7C15, 9
+    z = O.rand_normal([n], sx, sy).numpy()
+    for p in range((n + 1) // 2):
+        u1, u2 = u(sx + 2 * p, sy), u(sx + 2 * p + 1, sy)
+        r = math.sqrt(-2.0 * math.log(u1))
+        want = [r * math.cos(2 * math.pi * u2), r * math.sin(2 * math.pi * u2)]
+        for j in range(2):
+            if 2 * p + j < n:
+                assert abs(float(z[2 * p + j]) - want[j]) < 2e-6 * (1.0 + r), (p, j, z[2 * p + j], want[j])
+    # closed form: u2 = 0 would give (r, 0); here the invariant z1^2 + z2^2 = -2 ln u1 holds for every full pair
+    for p in range(n // 2):
+        assert abs(float(z[2 * p]) ** 2 + float(z[2 * p + 1]) ** 2 + 2.0 * math.log(u(sx + 2 * p, sy))) < 1e-5
+
+
+def test_scatter_against_explicit_loops():
+    """core.rs:764-833: for every element of `ind` (coordinates c): y[c with c[axis] := ind[c]] += x[c], y zero-filled
+    first; duplicates accumulate.  Nested Python loops on a rank-3 case with duplicate targets along the axis."""
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((3, 4, 5)).astype(np.float32)
+    for axis, out_ext in ((1, [3, 6, 5]), (0, [4, 4, 5]), (2, [3, 4, 7])):
+        ind = rng.integers(0, out_ext[axis], (3, 4, 5)).astype(np.uint32)
+        want = np.zeros(out_ext, np.float64)
+        for i in range(3):
+            for j in range(4):
+                for k in range(5):
+                    c = [i, j, k]
+                    c[axis] = int(ind[i, j, k])
+                    want[tuple(c)] += float(x[i, j, k])
+        got = O.scatter(T(x), T(ind), axis, out_ext).numpy()
+        close(got, want, 1e-5)
+        assert np.array_equal(got == 0, want == 0)  # untouched elements are exactly the zero fill
+    # an index tensor smaller than x along the axis (the gradient of a [B,1] gather, nn.rs:78-81): only ind's elements move
+    ind = rng.integers(0, 10, (3, 1, 5)).astype(np.uint32)
+    want = np.zeros((3, 10, 5))
+    for i in range(3):
+        for k in range(5):
+            want[i, ind[i, 0, k], k] += float(x[i, 0, k])
+    close(O.scatter(T(x[:, :1, :].copy()), T(ind), 1, [3, 10, 5]).numpy(), want, 1e-6)
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_gemm_batched_against_explicit_loops(ta, tb):
+    """gemm.rs:253-290 + matmul_direct.opencl:170-188: C[b,m,n] = sum_k op(A)[b,m,k] * op(B)[b,k,n] with the stored
+    layouts [b,K,M] / [b,N,K] under transposition; nested loops in float64 on a ragged case (a transposed-operand or
+    batch-stride mistake moves elements, which a tolerance of 1e-5 on O(1) values does not forgive)."""
+    rng = np.random.default_rng(17)
+    bt, m, k, n = 3, 5, 7, 4
+    a = rng.standard_normal((bt, k, m) if ta else (bt, m, k)).astype(np.float32)
+    b = rng.standard_normal((bt, n, k) if tb else (bt, k, n)).astype(np.float32)
+    want = np.zeros((bt, m, n))
+    for bi in range(bt):
+        for i in range(m):
+            for j in range(n):
+                for kk in range(k):
+                    av = a[bi, kk, i] if ta else a[bi, i, kk]
+                    bv = b[bi, j, kk] if tb else b[bi, kk, j]
+                    want[bi, i, j] += float(av) * float(bv)
+    close(O.gemm_batched(T(a), T(b), ta, tb).numpy(), want, 1e-5)

@@ -20,6 +20,15 @@ def say(*a):
     print("[case]", *a, flush=True)
 
 
+def device_free_bytes():
+    """Free device memory as the HIP runtime reports it (hipMemGetInfo), asked of the runtime directly: an
+    allocation made behind the context's own accounting (a stray hipMalloc in the call) would show here."""
+    hip = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(), C.c_size_t()
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
 def product(ctx, fn, a, b, bias, res, ta=False, tb=False):
     """relu(op(a).op(b) + bias) + res through one of the two rank-2 GEMM entry points."""
     lib = abi.lib()
@@ -29,9 +38,10 @@ def product(ctx, fn, a, b, bias, res, ta=False, tb=False):
     out = S.Tensor.uninit(ctx, [m, n])
     ac, bc, oc, biasc, resc = ta_.c(), tb_.c(), out.c(), tbias.c(), tres.c()
     epi = abi.sg_gemm_epilogue(1.0, abi.ACT_RELU, abi.ACT_NONE, C.pointer(biasc), C.pointer(resc))
-    before = ctx.mem_stats()
+    ctx.sync()
+    before = dict(ctx.mem_stats(), device_free=device_free_bytes())
     ctx.check(getattr(lib, fn)(ctx.handle, int(ta), int(tb), C.byref(ac), C.byref(bc), C.byref(oc), C.byref(epi)))
-    after = ctx.mem_stats()
+    after = dict(ctx.mem_stats(), device_free=device_free_bytes())
     return out.numpy(), before, after
 
 
@@ -52,6 +62,7 @@ def test_noalloc_gemm_matches_gemm_twice_second_smaller():
             exact(got, want, f"sg_gemm_noalloc {m}x{k}x{n}")
             # nothing taken from (or returned to) the context's allocator, nothing new held from the device
             assert after["used"] == before["used"] and after["reserved"] == before["reserved"]
+            assert after["device_free"] == before["device_free"], "the call changed the device's free memory"
             ref = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
             close(got, np.maximum(ref + bias, 0) + res, REL_GEMM, "vs float64")
     finally:
@@ -73,18 +84,23 @@ def test_noalloc_gemm_without_split_and_over_the_limit():
         # 4 tiles of 128x128 and K = 8192 split 32 ways: 32 * 256 * 256 * 4 B = 8 MiB fits; a product of
         # 1024 x 1024 outputs forced into 32 ranges (128 MiB of partial products) does not
         say("sg_gemm_noalloc over the scratch limit")
+        # (the library reads SAGE_GEMM_SPLITK once, when a context is created)
         import os
         os.environ["SAGE_GEMM_SPLITK"] = "32"
+        try:
+            forced = S.Context()
+        finally:
+            del os.environ["SAGE_GEMM_SPLITK"]
         try:
             a = rng.uniform(-1, 1, (1024, 4096)).astype(np.float32)
             b = rng.uniform(-1, 1, (4096, 1024)).astype(np.float32)
             with pytest.raises(abi.SageError, match="static scratch"):
-                product(ctx, "sg_gemm_noalloc", a, b, np.zeros(1024, np.float32), np.zeros((1024, 1024), np.float32))
+                product(forced, "sg_gemm_noalloc", a, b, np.zeros(1024, np.float32), np.zeros((1024, 1024), np.float32))
+            # the context still works after the refusal
+            got2, _, _ = product(forced, "sg_gemm_noalloc", a[:256, :512].copy(), b[:512, :128].copy(), np.zeros(128, np.float32),
+                                 np.zeros((256, 128), np.float32))
         finally:
-            del os.environ["SAGE_GEMM_SPLITK"]
-        # the context still works after the refusal
-        got2, _, _ = product(ctx, "sg_gemm_noalloc", a[:256, :512].copy(), b[:512, :128].copy(), np.zeros(128, np.float32),
-                             np.zeros((256, 128), np.float32))
+            forced.close()
         close(got2, np.maximum(a[:256, :512].astype(np.float64) @ b[:512, :128].astype(np.float64), 0), REL_GEMM, "after refusal")
     finally:
         ctx.close()

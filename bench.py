@@ -25,6 +25,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# `traffic` is not measured by this run: it is read, by kernel name, from the committed counter summaries under profiles/
+# (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same workload); it goes stale if the kernel changes and they are not re-collected
+TRAFFIC_SOURCE = "profiles/traffic_*.json (committed rocprofv3 --pmc summary of this workload, looked up by kernel name; not measured in this run)"
 
 
 def measured_traffic(kernel, workload):
@@ -401,6 +404,7 @@ def time_kernel_workload(ctx, name, steps, warmup, elements=None):
         achieved, peak, unit, bound = bytes_per / (per_ms * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s", "hbm"
     roof = {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
             "traffic": measured_traffic(label, name), "kernel": label, "avg_launch_ms": per_ms}
+    roof["traffic_source"] = TRAFFIC_SOURCE if roof["traffic"] is not None else None
     cfg = {"workload": name, "launches_per_step": launches, "buffer_sets": len(progs),
            "algorithmic_bytes_per_step": bytes_per, "flops_per_step": flops_per, "wall_ms_per_step": wall_ms}
     del progs
@@ -416,10 +420,15 @@ def hbm_rooflines(ctx, steps=2000, warmup=500):
     out = []
     for name in HBM_WORKLOADS:
         roof, cfg, _ = time_kernel_workload(ctx, name, steps, warmup)
-        out.append({"workload": name, "kernel": roof["kernel"], "bytes": cfg["algorithmic_bytes_per_step"],
-                    "avg_launch_ms": roof["avg_launch_ms"], "achieved": roof["achieved"], "unit": "GB/s",
-                    "frac": roof["frac"], "traffic": roof["traffic"], "launches_timed": steps})
         ctx.trim()
+        nbytes = cfg["algorithmic_bytes_per_step"]
+        # the bound that travels with the number: a plain streaming copy that moves the same number of bytes, same run
+        copy, _, _ = time_kernel_workload(ctx, "copy", steps, warmup, elements=max(1024, nbytes // 8 // 4 * 4))
+        ctx.trim()
+        out.append({"workload": name, "kernel": roof["kernel"], "bytes": nbytes,
+                    "avg_launch_ms": roof["avg_launch_ms"], "achieved": roof["achieved"], "unit": "GB/s",
+                    "frac": roof["frac"], "copy_frac": copy["frac"], "copy_avg_launch_ms": copy["avg_launch_ms"],
+                    "traffic": roof["traffic"], "traffic_source": TRAFFIC_SOURCE if roof["traffic"] is not None else None, "launches_timed": steps})
     return out
 
 
@@ -503,6 +512,7 @@ def main():
     ap.add_argument("--layers", type=int, default=12)
     ap.add_argument("--elements", type=int, default=None, help="copy workload: number of floats copied (default 64 Mi)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="bert at the headline shape: leave out the `configs` list (the other four configurations timed behind it)")
     ap.add_argument("--no-hbm-kernels", action="store_true", help="bert: leave out the roofline_hbm list (the fused map/reduce/row kernels timed after the model)")
     ap.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
                     help="replay the step as one HIP graph (auto = on; off: one host call per operator launch)")
@@ -522,20 +532,48 @@ def main():
         return run_kernel_workload(a)
 
     import sage_amd as S
+    ctx = S.Context(0)
+    res, keep = time_model(ctx, a.workload, a.variant, a.batch, a.seq, a.layers, a.steps, a.warmup, a.graph != "off")
+    headline = a.workload == "bert" and (a.batch, a.seq, a.layers, a.variant) == (32, 128, 12, "config")
+    if a.workload == "bert" and not a.no_hbm_kernels:
+        # the other half of the metric: the fused map / reduce / row kernels against the HBM peak, each beside a
+        # plain copy of the same number of bytes timed in this same run (what a launch of that size can reach)
+        ctx.trim()
+        res["roofline_hbm"] = hbm_rooflines(ctx)
+    if headline and not a.no_configs:
+        res["configs"] = other_configs(ctx, res)
+    if not a.no_cpu_baseline:
+        if a.workload == "resnet18":
+            res["cpu_baseline"] = cpu_baseline_resnet18(keep["model"], keep["arrays"], keep["x_host"])
+        elif a.batch * a.seq <= 4096:
+            res["cpu_baseline"] = cpu_baseline_whole_model(keep["bert"], a.variant, a.layers, keep["out0"])
+        else:
+            res["cpu_baseline"] = cpu_baseline(a.variant, a.batch, a.seq, 6)
+    print(json.dumps(res))
+
+
+def time_model(ctx, workload, variant, batch, seq, layers, steps, warmup, use_graph):
+    """Builds a model workload (bert | resnet18), runs `warmup` untimed and `steps` timed forward passes and times
+    the launches of its dominant GEMM instantiation with HIP event pairs on the context's stream.  Returns the
+    result line (metric, value, config, roofline) and what the CPU baseline needs (host arrays, first output).
+    Every device buffer of the model is released before returning."""
+    import sage_amd as S
     from sage_amd import abi
     lib = abi.lib()
-    ctx = S.Context(0)
     rng = np.random.default_rng(5)
-    if a.workload == "resnet18":
-        batch = a.batch if a.batch != 32 else 128
+    keep = {}
+    if workload == "resnet18":
+        batch = batch if batch != 32 else 128
         model, arrays, x_host, logits = build_resnet18(ctx, batch, rng)
+        keep.update(model=model, arrays=arrays, x_host=x_host)
     else:
-        batch = a.batch
-        bert = build_bert(ctx, a.variant, a.batch, a.seq, a.layers, rng, detail=True)
+        bert = build_bert(ctx, variant, batch, seq, layers, rng, detail=True)
         cfg, model, logits = bert["cfg"], bert["model"], bert["logits"]
+        keep.update(bert=bert)
     prog = S.Program(ctx, [logits])  # first evaluation: builds kernels, allocates every buffer
     ctx.sync()
     out0 = prog.outputs[0].numpy()
+    keep["out0"] = out0
     if not np.all(np.isfinite(out0)):
         raise SystemExit("non-finite model output")
 
@@ -545,6 +583,7 @@ def main():
     for i, name, flops, shape in gc:
         by_name.setdefault(name, []).append((i, flops, shape))
     dom = max(by_name, key=lambda n: sum(f for _, f, _ in by_name[n]))
+
     def new_event():
         e = C.c_void_p()
         ctx.check(lib.sg_event_create(ctx.handle, C.byref(e)))
@@ -556,86 +595,115 @@ def main():
     # the launches: every launch index is timed in steps/SAMPLE of the timed steps.
     SAMPLE = 6
     dom_calls = [i for i, _, _ in by_name[dom]]
-    pairs = [{i: (new_event(), new_event()) for j, i in enumerate(dom_calls) if j % SAMPLE == step % SAMPLE} for step in range(a.steps)]
+    pairs = [{i: (new_event(), new_event()) for j, i in enumerate(dom_calls) if j % SAMPLE == step % SAMPLE} for step in range(max(steps, SAMPLE))]
 
-    use_graph = a.graph != "off"
     if use_graph:
         prog.capture()
-    for _ in range(a.warmup):
+    for _ in range(warmup):
         prog.run()
     ctx.sync()
     t0 = time.perf_counter()
     if use_graph:
         # the timed region replays the graph; the dominant kernel's launches are timed with event
         # pairs in an eager replay of the same steps right behind it (events cannot bracket graph nodes)
-        for step in range(a.steps):
+        for step in range(steps):
             prog.run()
         ctx.sync()
         dt = time.perf_counter() - t0
-        for step in range(a.steps):
+        for step in range(len(pairs)):
             run_timed(ctx, prog, pairs[step])
         ctx.sync()
     else:
-        for step in range(a.steps):
+        for step in range(steps):
             run_timed(ctx, prog, pairs[step])
         ctx.sync()
         dt = time.perf_counter() - t0
+        for step in range(steps, len(pairs)):
+            run_timed(ctx, prog, pairs[step])
+        ctx.sync()
     flops_of = {i: f for i, f, _ in by_name[dom]}
     ms_of = {i: [] for i in flops_of}
-    for step in range(a.steps):
+    for step in range(len(pairs)):
         for i, (e0, e1) in pairs[step].items():
             ms = C.c_float()
             ctx.check(lib.sg_event_elapsed_ms(ctx.handle, e0, e1, C.byref(ms)))
             ms_of[i].append(ms.value)
-    ms_per_step = dt / a.steps * 1e3
+            lib.sg_event_destroy(ctx.handle, e0)
+            lib.sg_event_destroy(ctx.handle, e1)
+    ms_per_step = dt / steps * 1e3
 
     # Every launch index of the kernel counts once, whatever number of steps sampled it: the mean duration of
-    # each index first, then flops and time summed over the indices (all of them are sampled when steps >= SAMPLE).
+    # each index first, then flops and time summed over the indices (all of them are sampled: at least SAMPLE replays).
     sampled = [i for i in ms_of if ms_of[i]]
     n_timed = sum(len(ms_of[i]) for i in sampled)
     flops_per_launch = float(np.mean([flops_of[i] for i in sampled]))
     avg_ms = float(np.mean([np.mean(ms_of[i]) for i in sampled]))
     achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
     total_gemm_flops = sum(f for _, _, f, _ in gc)
-    if a.workload == "resnet18":
+    if workload == "resnet18":
         metric, unit = f"ResNet-18 fwd images/sec (b{batch},28x28x1,fp32)", "images/s"
         config = {"workload": f"resnet18_forward_b{batch}_28x28x1_fp32"}
+        traffic_key = f"resnet18_b{batch}_28x28"
     else:
-        metric, unit = f"BERT-base fwd seqs/sec (b{a.batch},s{a.seq},fp32)", "seqs/s"
-        config = {"workload": f"bert_base_forward_b{a.batch}_s{a.seq}_fp32", "variant": a.variant, "layers": a.layers,
+        metric, unit = f"BERT-base fwd seqs/sec (b{batch},s{seq},fp32)", "seqs/s"
+        config = {"workload": f"bert_base_forward_b{batch}_s{seq}_fp32", "variant": variant, "layers": layers,
                   "hidden": cfg.embed_dim, "heads": cfg.num_attention_heads, "ffn": cfg.hidden_dim, "vocab": cfg.num_vocabs,
-                  "segment_table_rows": 0 if a.variant == "reference" else 2}
+                  "segment_table_rows": 0 if variant == "reference" else 2}
+        traffic_key = f"bert_base_b{batch}_s{seq}" if layers == 12 and variant == "config" else None
     config.update({"replay": "hip_graph" if use_graph else "eager", "launches_per_step": len(prog.calls), "gemm_tflops_whole_step": total_gemm_flops / (ms_per_step * 1e-3) / 1e12})
+    traffic = measured_traffic(dom, traffic_key) if traffic_key else None
     res = {
         "metric": metric,
         "value": batch / (ms_per_step * 1e-3),
         "unit": unit,
-        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": config,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
-                     "traffic": measured_traffic(dom, f"bert_base_b{a.batch}_s{a.seq}") if a.workload == "bert" and a.layers == 12 and a.variant == "config" else None,
+                     "traffic": traffic, "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
                      "kernel": dom,
                      "launches_per_step": len(by_name[dom]), "launch_indices_sampled": len(sampled), "launches_timed": n_timed, "avg_launch_ms": avg_ms, "flops_per_launch": flops_per_launch,
                      "shapes_mnkb": sorted({s for _, _, s in by_name[dom]})},
     }
-    if a.workload == "bert" and not a.no_hbm_kernels:
-        # the other half of the metric: the fused map / reduce / row kernels against the HBM peak
-        if use_graph:
-            prog.release_graph()
-        del prog
-        ctx.trim()
-        res["roofline_hbm"] = hbm_rooflines(ctx)
-    if not a.no_cpu_baseline:
-        if a.workload == "resnet18":
-            res["cpu_baseline"] = cpu_baseline_resnet18(model, arrays, x_host)
-        elif a.batch * a.seq <= 4096:
-            res["cpu_baseline"] = cpu_baseline_whole_model(bert, a.variant, a.layers, out0)
-        else:
-            res["cpu_baseline"] = cpu_baseline(a.variant, a.batch, a.seq, 6)
-    print(json.dumps(res))
+    if use_graph:
+        prog.release_graph()
+    del prog, logits, model
+    if "bert" in keep:
+        for k in ("model", "logits", "hidden"):
+            keep["bert"].pop(k, None)
+    import gc as _gc
+    _gc.collect()
+    ctx.trim()
+    return res, keep
+
+
+def other_configs(ctx, headline):
+    """The other four benchmark configurations, timed in the same run behind the headline: softmax cross-entropy
+    [8192,1024] (one fused launch), the 4096^3 GEMM with its bias epilogue, ResNet-18 forward at b128 and the full
+    BERT-base forward at b64 x s512.  One entry each: workload, ms_per_step, value/unit and the roofline of its
+    dominant kernel."""
+    out = []
+    ce = next(e for e in headline["roofline_hbm"] if e["workload"] == "softmax_ce") if "roofline_hbm" in headline else None
+    if ce is not None:
+        out.append({"workload": "softmax_cross_entropy_8192x1024_fp32", "ms_per_step": ce["avg_launch_ms"], "value": 8192 / (ce["avg_launch_ms"] * 1e-3), "unit": "rows/s",
+                    "roofline": {"bound": "hbm", "kernel": ce["kernel"], "frac": ce["frac"], "copy_frac": ce["copy_frac"], "avg_launch_ms": ce["avg_launch_ms"],
+                                 "bytes_per_launch": ce["bytes"], "achieved": ce["achieved"], "unit": "GB/s"}})
+    roof, cfg, _ = time_kernel_workload(ctx, "gemm_bias", 200, 30)
+    out.append({"workload": "gemm_bias_4096x4096x4096_fp32", "ms_per_step": roof["avg_launch_ms"], "value": roof["achieved"], "unit": "TFLOP/s",
+                "roofline": {"bound": "mfma", "kernel": roof["kernel"], "frac": roof["frac"], "avg_launch_ms": roof["avg_launch_ms"],
+                             "flops_per_launch": cfg["flops_per_step"], "achieved": roof["achieved"], "unit": "TFLOP/s", "launches_timed": 200}})
+    ctx.trim()
+    for workload, batch, seq, steps, warmup in (("resnet18", 128, 0, 50, 10), ("bert", 64, 512, 6, 2)):
+        r, _ = time_model(ctx, workload, "config", batch, seq, 12, steps, warmup, True)
+        rf = r["roofline"]
+        out.append({"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "value": r["value"], "unit": r["unit"], "steps": steps,
+                    "launches_per_step": r["config"]["launches_per_step"], "gemm_tflops_whole_step": r["config"]["gemm_tflops_whole_step"],
+                    "roofline": {"bound": "mfma", "kernel": rf["kernel"], "frac": rf["frac"], "avg_launch_ms": rf["avg_launch_ms"],
+                                 "flops_per_launch": rf["flops_per_launch"], "achieved": rf["achieved"], "unit": "TFLOP/s",
+                                 "launches_timed": rf["launches_timed"], "shapes_mnkb": rf["shapes_mnkb"]}})
+    return out
 
 
 if __name__ == "__main__":

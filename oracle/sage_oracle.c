@@ -655,12 +655,16 @@ int or_im2col(const sg_tensor *x, const sg_tensor *out, const int32_t ker[2], co
 /* ---------------------------------------------------------------------------------------------
  * Col2im::compute (conv.rs:405-500).  Work-item = (img_y, img_x, c); the batch and the contributing
  * columns are looped inside it, col_x outer and col_y inner (the order of the float additions).
- * The reference tests ker_x against dilation_h and ker_y against dilation_w (conv.rs:463-465);
- * kept as is, it only matters when the two dilations differ.  Pairs are {w, h}.
+ * The reference tests ker_x against dilation_h and ker_y against dilation_w (conv.rs:463-465) and
+ * divides by them; kept as is.  Where the two dilations differ (and the kernel has more than one tap)
+ * the tap indices that come out of that lie outside [0, ker): the reference's kernel then reads
+ * entries of other taps or past the end of its buffer, i.e. it defines no result; this restatement
+ * refuses such a geometry (OR_ERR) instead of reading out of bounds.  Pairs are {w, h}.
  * ------------------------------------------------------------------------------------------- */
 int or_col2im(const sg_tensor *x, const sg_tensor *out, const int32_t ker[2], const int32_t stride[2],
               const int32_t pad[2], const int32_t dil[2]) {
     if (x->rank != 6 || out->rank != 4) return OR_ERR;
+    if (dil[0] != dil[1] && (ker[0] > 1 || ker[1] > 1)) return OR_ERR; /* undefined in the reference, see above */
     int batch = (int)x->extents[0], col_h = (int)x->extents[1], col_w = (int)x->extents[2], chan = (int)x->extents[5];
     int img_h = (int)out->extents[1], img_w = (int)out->extents[2];
     int ker_w = ker[0], ker_h = ker[1], stride_w = stride[0], stride_h = stride[1];

@@ -10,18 +10,56 @@
 
 namespace {
 
+// Index space of a kernel after the host has collapsed it: extents with their multiply-high magic numbers (no
+// hardware division on the device; the outermost axis needs none) and up to three stride sets over them.
 struct Dims {
     int n;
     uint32_t ext[SG_MAX_RANK];
-    uint32_t stride[SG_MAX_RANK];
+    sg_fastdiv div[SG_MAX_RANK];
+    uint32_t stride[3][SG_MAX_RANK];
 };
 
-Dims dims_of(const int64_t *ext, const int64_t *st, int rank) {
-    Dims d;
-    d.n = rank;
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, sg_fastdiv d) { return (__umulhi(n, d.magic) + n) >> d.shift; }
+
+// Collapses the index space `ext` walked by n_sets stride sets: axes of extent 1 vanish and two neighbouring axes
+// merge when every stride set steps through them like through one axis (stride[a] == ext[a+1] * stride[a+1]).
+// `keep` (or -1) names an axis that must stay on its own (the gather / scatter axis, whose coordinate is replaced
+// by an index); *keep_out receives its position after the collapse.  A dense tensor becomes one axis, a row gather two.
+Dims collapse(int rank, const int64_t *ext, int n_sets, const int64_t *const *strides, int keep, int *keep_out) {
+    int64_t e[SG_MAX_RANK], st[3][SG_MAX_RANK];
+    bool is_keep[SG_MAX_RANK];
+    int n = 0;
+    for (int a = 0; a < rank; ++a) {
+        if (ext[a] == 1 && a != keep) continue;
+        const bool merge = n > 0 && a != keep && !is_keep[n - 1] && [&] {
+            for (int k = 0; k < n_sets; ++k)
+                if (st[k][n - 1] != ext[a] * strides[k][a]) return false;
+            return true;
+        }();
+        if (merge) {
+            e[n - 1] *= ext[a];
+            for (int k = 0; k < n_sets; ++k) st[k][n - 1] = strides[k][a];
+        } else {
+            e[n] = ext[a];
+            for (int k = 0; k < n_sets; ++k) st[k][n] = strides[k][a];
+            is_keep[n] = a == keep;
+            ++n;
+        }
+    }
+    if (n == 0) {  // a single element
+        e[0] = 1;
+        for (int k = 0; k < n_sets; ++k) st[k][0] = 0;
+        is_keep[0] = false;
+        n = 1;
+    }
+    Dims d{};
+    d.n = n;
+    if (keep_out) *keep_out = -1;
     for (int i = 0; i < SG_MAX_RANK; ++i) {
-        d.ext[i] = i < rank ? (uint32_t)ext[i] : 1;
-        d.stride[i] = i < rank ? (uint32_t)st[i] : 0;
+        d.ext[i] = i < n ? (uint32_t)e[i] : 1u;
+        d.div[i] = sg_make_fastdiv(d.ext[i]);
+        for (int k = 0; k < 3; ++k) d.stride[k][i] = i < n && k < n_sets ? (uint32_t)st[k][i] : 0u;
+        if (i < n && is_keep[i] && keep_out) *keep_out = i;
     }
     return d;
 }
@@ -32,22 +70,23 @@ __global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t *__restrict__ p,
     for (; i < n; i += step) p[i] = v;
 }
 
-// out[gid] = x[x_off + sum_i (i == axis ? ind[...] : c_i) * xstride_i]; c from ind's extents.
+// out[gid] = x[x_off + sum_i (i == axis ? ind[...] : c_i) * xstride_i]; c from ind's extents (collapsed on the host).
+// Stride set 0 walks ind, set 1 walks x.
 __global__ void __launch_bounds__(256) gather_kernel(const uint32_t *__restrict__ x, const uint32_t *__restrict__ ind,
-                                                     uint32_t *__restrict__ y, uint32_t n, Dims idims, Dims xdims, int axis,
+                                                     uint32_t *__restrict__ y, uint32_t n, Dims d, int axis,
                                                      uint32_t x_off, uint32_t ind_off) {
     uint32_t gid = blockIdx.x * 256u + threadIdx.x;
     if (gid >= n) return;
-    uint32_t rem = gid, ioff = ind_off, xo = x_off, caxis_stride = xdims.stride[axis];
-    for (int a = idims.n - 1; a >= 0; --a) {
-        uint32_t q = rem / idims.ext[a];
-        uint32_t c = rem - q * idims.ext[a];
+    uint32_t rem = gid, ioff = ind_off, xo = x_off;
+    for (int a = d.n - 1; a >= 0; --a) {
+        const uint32_t q = a ? fdiv(rem, d.div[a]) : 0u;
+        const uint32_t c = rem - q * d.ext[a];
         rem = q;
-        ioff += c * idims.stride[a];
-        if (a != axis) xo += c * xdims.stride[a];
+        ioff += c * d.stride[0][a];
+        if (a != axis) xo += c * d.stride[1][a];
     }
     const uint32_t target = ind[ioff];
-    y[gid] = x[xo + target * caxis_stride];
+    y[gid] = x[xo + target * d.stride[1][axis]];
 }
 
 // Row gather: x [V, E] with unit inner stride, one index per output row (the index tensor is expanded along the
@@ -59,49 +98,67 @@ __global__ void __launch_bounds__(256) gather_rows_kernel(const uint32_t *__rest
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
     if (gid >= n_vec) return;
-    const uint32_t row = (__umulhi(gid, d_row.magic) + gid) >> d_row.shift, c = gid - row * vec_per_row;
+    const uint32_t row = fdiv(gid, d_row), c = gid - row * vec_per_row;
     const uint32_t target = ind[ind_off + row * ind_row_stride];
     *reinterpret_cast<u32x4 *>(y + (size_t)gid * 4u) = *reinterpret_cast<const u32x4 *>(x + x_off + (size_t)target * x_row_stride + c * 4u);
 }
 
 template <class T>
 __global__ void __launch_bounds__(256) scatter_add_kernel(const T *__restrict__ x, const uint32_t *__restrict__ ind, T *__restrict__ y,
-                                                          uint32_t n, Dims idims, Dims xdims, Dims ydims, int axis, uint32_t x_off,
-                                                          uint32_t ind_off) {
+                                                          uint32_t n, Dims d, int axis, uint32_t x_off, uint32_t ind_off) {
+    // stride set 0 walks ind, 1 walks x, 2 walks y
     uint32_t gid = blockIdx.x * 256u + threadIdx.x;
     if (gid >= n) return;
     uint32_t rem = gid, ioff = ind_off, xo = x_off, yo = 0;
-    for (int a = idims.n - 1; a >= 0; --a) {
-        uint32_t q = rem / idims.ext[a];
-        uint32_t c = rem - q * idims.ext[a];
+    for (int a = d.n - 1; a >= 0; --a) {
+        const uint32_t q = a ? fdiv(rem, d.div[a]) : 0u;
+        const uint32_t c = rem - q * d.ext[a];
         rem = q;
-        ioff += c * idims.stride[a];
-        xo += c * xdims.stride[a];
-        if (a != axis) yo += c * ydims.stride[a];
+        ioff += c * d.stride[0][a];
+        xo += c * d.stride[1][a];
+        if (a != axis) yo += c * d.stride[2][a];
     }
-    yo += ind[ioff] * ydims.stride[axis];
+    yo += ind[ioff] * d.stride[2][axis];
     atomicAdd(&y[yo], x[xo]);
 }
 
 // strided window copy: y[ydims(c)] = x[xdims(c)], c enumerates x's extents
 __global__ void __launch_bounds__(256) window_copy_kernel(const uint32_t *__restrict__ x, uint32_t *__restrict__ y, uint32_t n,
-                                                          Dims xdims, Dims ydims, uint32_t x_off, uint32_t y_off) {
+                                                          Dims d, uint32_t x_off, uint32_t y_off) {
+    // stride set 0 walks x, 1 walks y
     uint32_t gid = blockIdx.x * 256u + threadIdx.x;
     if (gid >= n) return;
     uint32_t rem = gid, xo = x_off, yo = y_off;
-    for (int a = xdims.n - 1; a >= 0; --a) {
-        uint32_t q = rem / xdims.ext[a];
-        uint32_t c = rem - q * xdims.ext[a];
+    for (int a = d.n - 1; a >= 0; --a) {
+        const uint32_t q = a ? fdiv(rem, d.div[a]) : 0u;
+        const uint32_t c = rem - q * d.ext[a];
         rem = q;
-        xo += c * xdims.stride[a];
-        yo += c * ydims.stride[a];
+        xo += c * d.stride[0][a];
+        yo += c * d.stride[1][a];
     }
     y[yo] = x[xo];
 }
 
 struct Im2colP {
     int batch, chan, img_w, img_h, col_w, col_h, ker_w, ker_h, stride_w, stride_h, pad_w, pad_h, dil_w, dil_h;
+    // magic numbers for the decompositions below, set by finish(): channel groups per pixel, column / image / kernel
+    // extents, and the strides (col2im divides by them)
+    sg_fastdiv d_cv, d_col_w, d_col_h, d_ker_w, d_ker_h, d_img_w, d_img_h, d_stride_w, d_stride_h;
+    void finish(int vec) {
+        d_cv = sg_make_fastdiv((uint32_t)(chan / vec));
+        d_col_w = sg_make_fastdiv((uint32_t)col_w); d_col_h = sg_make_fastdiv((uint32_t)col_h);
+        d_ker_w = sg_make_fastdiv((uint32_t)ker_w); d_ker_h = sg_make_fastdiv((uint32_t)ker_h);
+        d_img_w = sg_make_fastdiv((uint32_t)img_w); d_img_h = sg_make_fastdiv((uint32_t)img_h);
+        d_stride_w = sg_make_fastdiv((uint32_t)stride_w); d_stride_h = sg_make_fastdiv((uint32_t)stride_h);
+    }
 };
+
+// rem -> (rem / d, rem % d) by multiply-high
+__device__ __forceinline__ uint32_t split(uint32_t &rem, uint32_t d, sg_fastdiv m) {
+    const uint32_t q = fdiv(rem, m), r = rem - q * d;
+    rem = q;
+    return r;
+}
 
 // Pooling without the column tensor: out[n, oy, ox, c] = reduce over (ky, kx) of the window the reference's
 // max_pool_2d / avg_pool_2d first copy out with im2col and then reduce over axes [3, 4] (conv.rs:143-165).
@@ -113,11 +170,10 @@ __global__ void __launch_bounds__(256) pool2d_kernel(const float *__restrict__ i
                                                      int op, int ref_zero) {
     uint32_t gid = blockIdx.x * 256u + threadIdx.x;
     if (gid >= n_vec) return;
-    const uint32_t cv = p.chan / VEC;
     uint32_t rem = gid;
-    const uint32_t c = (rem % cv) * VEC; rem /= cv;
-    const uint32_t ox = rem % p.col_w; rem /= p.col_w;
-    const uint32_t oy = rem % p.col_h; rem /= p.col_h;
+    const uint32_t c = split(rem, (uint32_t)p.chan / VEC, p.d_cv) * VEC;
+    const uint32_t ox = split(rem, (uint32_t)p.col_w, p.d_col_w);
+    const uint32_t oy = split(rem, (uint32_t)p.col_h, p.d_col_h);
     const uint32_t n = rem;
     const float start = ref_zero ? 0.0f : (op == SG_R_SUM ? 0.0f : op == SG_R_PROD ? 1.0f : op == SG_R_MAX ? -__builtin_inff() : __builtin_inff());
     float acc[VEC];
@@ -167,14 +223,13 @@ template <int VEC>
 __global__ void __launch_bounds__(256) im2col_kernel(const float *__restrict__ img, float *__restrict__ col, uint32_t n_vec, Im2colP p) {
     uint32_t gid = blockIdx.x * 256u + threadIdx.x;
     if (gid >= n_vec) return;
-    const uint32_t cv = p.chan / VEC;
     uint32_t rem = gid;
-    uint32_t c = (rem % cv) * VEC; rem /= cv;
-    uint32_t kx = rem % p.ker_w; rem /= p.ker_w;
-    uint32_t ky = rem % p.ker_h; rem /= p.ker_h;
-    uint32_t ox = rem % p.col_w; rem /= p.col_w;
-    uint32_t oy = rem % p.col_h; rem /= p.col_h;
-    uint32_t n = rem;
+    const uint32_t c = split(rem, (uint32_t)p.chan / VEC, p.d_cv) * VEC;
+    const uint32_t kx = split(rem, (uint32_t)p.ker_w, p.d_ker_w);
+    const uint32_t ky = split(rem, (uint32_t)p.ker_h, p.d_ker_h);
+    const uint32_t ox = split(rem, (uint32_t)p.col_w, p.d_col_w);
+    const uint32_t oy = split(rem, (uint32_t)p.col_h, p.d_col_h);
+    const uint32_t n = rem;
     const int ix = (int)ox * p.stride_w - p.pad_w + (int)kx * p.dil_w;
     const int iy = (int)oy * p.stride_h - p.pad_h + (int)ky * p.dil_h;
     const bool inside = ix >= 0 && ix < p.img_w && iy >= 0 && iy < p.img_h;
@@ -187,42 +242,42 @@ __global__ void __launch_bounds__(256) im2col_kernel(const float *__restrict__ i
     }
 }
 
-// Col2im::compute (conv.rs:405-500): img[n,y,x,c] = sum of the column entries that im2col copied
-// from that pixel.  One thread per output element (the reference loops the batch inside a work-item);
-// the additions run col_x outer, col_y inner, as the reference's, so the sum is bit-identical to a
-// sequential restatement.  The reference tests ker_x against dilation_h and ker_y against dilation_w
-// (conv.rs:463-465); kept, it only matters when the two dilations differ.
-// VEC = 4: a thread sums four consecutive channels (16-byte loads, one 16-byte store); each channel's additions
-// keep their order.
+// Col2im::compute (conv.rs:405-500), the adjoint of im2col: out[n, y, x, c] is the sum of every column entry that
+// im2col copied from that pixel.  Tap-centric: tap (ky, kx) of output cell (oy, ox) was read from pixel
+// (oy*stride_h - pad_h + ky*dil_h, ox*stride_w - pad_w + kx*dil_w), so for each tap the one cell that read THIS pixel
+// through it is found by solving for (oy, ox): the remainder of (y + pad_h - ky*dil_h) by stride_h must vanish and
+// the quotient must be a row of the column tensor, likewise across.  One thread per VEC channels of a pixel; the
+// divisions by the strides are multiply-highs, nothing in the loop divides.
+// Order of the float additions: the reference's work-item walks the cells with ox ascending outside and oy
+// ascending inside; a larger ox means a smaller kx, so the taps run kx descending outside, ky descending inside and
+// the sum is bit-identical to the reference's.  Where the two dilations differ the reference's kernel takes its
+// tap indices from the wrong dilation (conv.rs:463-465) and reads entries of other taps or past its buffer: it
+// defines no result there; this kernel returns the adjoint.
 template <int VEC>
 __global__ void __launch_bounds__(256) col2im_kernel(const float *__restrict__ col, float *__restrict__ img, uint32_t n_out, Im2colP p) {
     typedef float vec_t __attribute__((ext_vector_type(VEC)));
     const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
     if (gid >= n_out) return;
-    const uint32_t cv = p.chan / VEC;  // channel groups per pixel
-    const int c = (gid % cv) * VEC;
-    uint32_t t = gid / cv;
-    const int img_x = t % p.img_w;
-    t /= p.img_w;
-    const int img_y = t % p.img_h;
-    const int n = t / p.img_h;
-    const int img_x_pad = img_x + p.pad_w, img_y_pad = img_y + p.pad_h;
-    const int ker_ew = (p.ker_w - 1) * p.dil_w + 1, ker_eh = (p.ker_h - 1) * p.dil_h + 1;
-    const int col_x_start = img_x_pad < ker_ew ? 0 : (img_x_pad - ker_ew) / p.stride_w + 1;
-    const int col_y_start = img_y_pad < ker_eh ? 0 : (img_y_pad - ker_eh) / p.stride_h + 1;
-    const int col_x_end = min(img_x_pad / p.stride_w + 1, p.col_w);
-    const int col_y_end = min(img_y_pad / p.stride_h + 1, p.col_h);
+    uint32_t rem = gid;
+    const uint32_t c = split(rem, (uint32_t)p.chan / VEC, p.d_cv) * VEC;
+    const uint32_t x = split(rem, (uint32_t)p.img_w, p.d_img_w);
+    const uint32_t y = split(rem, (uint32_t)p.img_h, p.d_img_h);
+    const uint32_t n = rem;
     const float *cb = col + (size_t)n * p.col_h * p.col_w * p.ker_h * p.ker_w * p.chan + c;
     vec_t val = 0.0f;
-    for (int col_x = col_x_start; col_x < col_x_end; ++col_x)
-        for (int col_y = col_y_start; col_y < col_y_end; ++col_y) {
-            int ker_x = img_x_pad - col_x * p.stride_w, ker_y = img_y_pad - col_y * p.stride_h;
-            if (ker_x % p.dil_h == 0 && ker_y % p.dil_w == 0) {
-                ker_x /= p.dil_h;
-                ker_y /= p.dil_w;
-                val += *reinterpret_cast<const vec_t *>(cb + (size_t)(((col_y * p.col_w + col_x) * p.ker_h + ker_y) * p.ker_w + ker_x) * p.chan);
-            }
+    for (int kx = p.ker_w - 1; kx >= 0; --kx) {
+        const int ax = (int)x + p.pad_w - kx * p.dil_w;  // = ox * stride_w for the cell that read this pixel through kx
+        if (ax < 0) continue;
+        const uint32_t ox = fdiv((uint32_t)ax, p.d_stride_w);
+        if (ox * (uint32_t)p.stride_w != (uint32_t)ax || ox >= (uint32_t)p.col_w) continue;
+        for (int ky = p.ker_h - 1; ky >= 0; --ky) {
+            const int ay = (int)y + p.pad_h - ky * p.dil_h;
+            if (ay < 0) continue;
+            const uint32_t oy = fdiv((uint32_t)ay, p.d_stride_h);
+            if (oy * (uint32_t)p.stride_h != (uint32_t)ay || oy >= (uint32_t)p.col_h) continue;
+            val += *reinterpret_cast<const vec_t *>(cb + (size_t)(((oy * p.col_w + ox) * p.ker_h + ky) * p.ker_w + kx) * p.chan);
         }
+    }
     *reinterpret_cast<vec_t *>(img + (size_t)gid * VEC) = val;
 }
 
@@ -264,9 +319,11 @@ extern "C" int sg_gather(sg_ctx *ctx, int axis, const sg_tensor *x, const sg_ten
         SG_CHECK_LAUNCH(ctx, "gather (rows)");
         return SG_OK;
     }
-    Dims idims = dims_of(ind->extents, ind->strides, ind->rank), xdims = dims_of(x->extents, x->strides, x->rank);
+    int axis_c = 0;
+    const int64_t *sets[2] = {ind->strides, x->strides};
+    const Dims d = collapse(ind->rank, ind->extents, 2, sets, axis, &axis_c);
     hipLaunchKernelGGL(gather_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, (const uint32_t *)x->base, (const uint32_t *)ind->base,
-                       (uint32_t *)out->base + out->offset, n, idims, xdims, axis, (uint32_t)x->offset, (uint32_t)ind->offset);
+                       (uint32_t *)out->base + out->offset, n, d, axis_c, (uint32_t)x->offset, (uint32_t)ind->offset);
     SG_CHECK_LAUNCH(ctx, "gather");
     return SG_OK;
 }
@@ -292,15 +349,16 @@ extern "C" int sg_scatter(sg_ctx *ctx, int axis, const sg_tensor *x, const sg_te
     }
     if ((rc = sg_fill_u32(ctx, (uint32_t *)out->base + out->offset, 0u, (uint64_t)sg_numel(out))) != SG_OK) return rc;
     const uint32_t n = (uint32_t)sg_numel(ind);
-    Dims idims = dims_of(ind->extents, ind->strides, ind->rank), xdims = dims_of(x->extents, x->strides, x->rank),
-         ydims = dims_of(out->extents, out->strides, out->rank);
+    int axis_c = 0;
+    const int64_t *sets[3] = {ind->strides, x->strides, out->strides};
+    const Dims d = collapse(ind->rank, ind->extents, 3, sets, axis, &axis_c);
     dim3 grid((n + 255) / 256);
     if (x->dtype == SG_FLOAT)
         hipLaunchKernelGGL((scatter_add_kernel<float>), grid, dim3(256), 0, ctx->stream, (const float *)x->base, (const uint32_t *)ind->base,
-                           (float *)out->base + out->offset, n, idims, xdims, ydims, axis, (uint32_t)x->offset, (uint32_t)ind->offset);
+                           (float *)out->base + out->offset, n, d, axis_c, (uint32_t)x->offset, (uint32_t)ind->offset);
     else
         hipLaunchKernelGGL((scatter_add_kernel<unsigned>), grid, dim3(256), 0, ctx->stream, (const unsigned *)x->base, (const uint32_t *)ind->base,
-                           (unsigned *)out->base + out->offset, n, idims, xdims, ydims, axis, (uint32_t)x->offset, (uint32_t)ind->offset);
+                           (unsigned *)out->base + out->offset, n, d, axis_c, (uint32_t)x->offset, (uint32_t)ind->offset);
     SG_CHECK_LAUNCH(ctx, "scatter");
     return SG_OK;
 }
@@ -319,9 +377,10 @@ extern "C" int sg_unslice(sg_ctx *ctx, int axis, int64_t start, const sg_tensor 
     }
     if ((rc = sg_fill_u32(ctx, (uint32_t *)out->base + out->offset, 0u, (uint64_t)sg_numel(out))) != SG_OK) return rc;
     const uint32_t n = (uint32_t)sg_numel(x);
-    Dims xdims = dims_of(x->extents, x->strides, x->rank), ydims = dims_of(x->extents, out->strides, x->rank);
+    const int64_t *sets[2] = {x->strides, out->strides};
+    const Dims d = collapse(x->rank, x->extents, 2, sets, -1, nullptr);
     hipLaunchKernelGGL(window_copy_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, (const uint32_t *)x->base, (uint32_t *)out->base, n,
-                       xdims, ydims, (uint32_t)x->offset, (uint32_t)(out->offset + start * out->strides[axis]));
+                       d, (uint32_t)x->offset, (uint32_t)(out->offset + start * out->strides[axis]));
     SG_CHECK_LAUNCH(ctx, "unslice");
     return SG_OK;
 }
@@ -347,9 +406,10 @@ extern "C" int sg_concat(sg_ctx *ctx, int axis, const sg_tensor *in, int n_in, c
     for (int k = 0; k < n_in; ++k) {
         const sg_tensor *v = &in[k];
         const uint32_t n = (uint32_t)sg_numel(v);
-        Dims xdims = dims_of(v->extents, v->strides, v->rank), ydims = dims_of(v->extents, out->strides, v->rank);
+        const int64_t *sets[2] = {v->strides, out->strides};
+        const Dims d = collapse(v->rank, v->extents, 2, sets, -1, nullptr);
         hipLaunchKernelGGL(window_copy_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, (const uint32_t *)v->base, (uint32_t *)out->base, n,
-                           xdims, ydims, (uint32_t)v->offset, (uint32_t)(out->offset + at * out->strides[axis]));
+                           d, (uint32_t)v->offset, (uint32_t)(out->offset + at * out->strides[axis]));
         SG_CHECK_LAUNCH(ctx, "concat");
         at += v->extents[axis];
     }
@@ -385,6 +445,7 @@ extern "C" int sg_im2col(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, 
     float *col = (float *)out->base + out->offset;
     const int64_t total = sg_numel(out);
     const bool vec = p.chan % 4 == 0 && ((uintptr_t)img % 16 == 0) && ((uintptr_t)col % 16 == 0);
+    p.finish(vec ? 4 : 1);
     if (vec) {
         const uint32_t n = (uint32_t)(total / 4);
         hipLaunchKernelGGL((im2col_kernel<4>), dim3((n + 255) / 256), dim3(256), 0, ctx->stream, img, col, n, p);
@@ -426,6 +487,7 @@ extern "C" int sg_pool2d(sg_ctx *ctx, int op, int init_mode, const sg_tensor *x,
     const int64_t total = sg_numel(out);
     const int ref_zero = init_mode == SG_INIT_REF_ZERO;
     const bool vec = p.chan % 4 == 0 && ((uintptr_t)img % 16 == 0) && ((uintptr_t)dst % 16 == 0);
+    p.finish(vec ? 4 : 1);
     if (vec) {
         const uint32_t n = (uint32_t)(total / 4);
         hipLaunchKernelGGL((pool2d_kernel<4>), dim3((n + 255) / 256), dim3(256), 0, ctx->stream, img, dst, n, p, op, ref_zero);
@@ -447,7 +509,7 @@ extern "C" int sg_col2im(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, 
     if (x->rank != 6 || out->rank != 4) return sg_fail(ctx, SG_ERR_SHAPE, "sg_col2im: x must be [N,OH,OW,KH,KW,C], out [N,H,W,C] (conv.rs:243)");
     if (!sg_is_dense(x) || !sg_is_dense(out)) return sg_fail(ctx, SG_ERR_SHAPE, "sg_col2im: x and out must be dense (conv.rs:244)");
     for (int i = 0; i < 2; ++i)
-        // dilation 0 would divide by zero in the reference's kernel (conv.rs:463-465): refused
+        // dilation 0 divides by zero in the reference's kernel (conv.rs:463-465): refused
         if (ker[i] < 1 || stride[i] < 1 || pad[i] < 0 || dil[i] < 1) return sg_fail(ctx, SG_ERR_ARG, "sg_col2im: bad geometry");
     Im2colP p;
     p.batch = (int)out->extents[0]; p.img_h = (int)out->extents[1]; p.img_w = (int)out->extents[2]; p.chan = (int)out->extents[3];
@@ -460,7 +522,9 @@ extern "C" int sg_col2im(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *out, 
     if (total >= (1ll << 32) || sg_numel(x) >= (1ll << 32)) return sg_fail(ctx, SG_ERR_SHAPE, "sg_col2im: more than 2^32 elements");
     const float *col = (const float *)x->base + x->offset;
     float *img = (float *)out->base + out->offset;
-    if (p.chan % 4 == 0 && (uintptr_t)col % 16 == 0 && (uintptr_t)img % 16 == 0)
+    const bool vec = p.chan % 4 == 0 && (uintptr_t)col % 16 == 0 && (uintptr_t)img % 16 == 0;
+    p.finish(vec ? 4 : 1);
+    if (vec)
         hipLaunchKernelGGL((col2im_kernel<4>), dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, ctx->stream, col, img, (uint32_t)(total / 4), p);
     else
         hipLaunchKernelGGL((col2im_kernel<1>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, col, img, (uint32_t)total, p);

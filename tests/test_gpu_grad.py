@@ -67,14 +67,28 @@ def test_col2im_reference_vector(ctx, golden):
 @pytest.mark.parametrize("n,h,w,c,ker,stride,pad,dil", [
     (2, 9, 7, 3, [3, 3], [1, 1], [1, 1], [1, 1]), (3, 14, 14, 8, [3, 3], [2, 2], [1, 1], [1, 1]),
     (1, 28, 28, 1, [7, 7], [2, 2], [3, 3], [1, 1]), (2, 8, 8, 4, [1, 1], [2, 2], [0, 0], [1, 1]),
-    (2, 11, 10, 2, [3, 2], [2, 1], [0, 1], [2, 2]), (1, 7, 7, 64, [3, 3], [1, 1], [1, 1], [1, 1])])
+    (2, 11, 10, 2, [3, 2], [2, 1], [0, 1], [2, 2]), (1, 7, 7, 64, [3, 3], [1, 1], [1, 1], [1, 1]),
+    (2, 12, 9, 8, [5, 3], [3, 2], [2, 1], [1, 1]), (1, 6, 5, 4, [2, 2], [3, 3], [0, 0], [1, 1]),  # stride above the kernel: pixels no tap reads
+    # two different dilations: the reference's kernel defines no result (it takes tap indices from the wrong dilation,
+    # conv.rs:463-465), the oracle refuses, the product returns the adjoint (checked by the identity below)
+    (2, 11, 10, 4, [3, 2], [1, 2], [1, 1], [1, 2]), (1, 9, 12, 3, [2, 3], [2, 1], [2, 0], [3, 1])])
 def test_col2im_vs_oracle_and_adjoint(ctx, n, h, w, c, ker, stride, pad, dil):
     say("col2im", n, h, w, c, ker, stride, pad, dil)
     rng = np.random.default_rng(h * 100 + w)
     ow, oh = V.conv_size([w, h], ker, stride, pad, dil)
     col = rng.standard_normal((n, oh, ow, ker[1], ker[0], c)).astype(np.float32)
     y = V.col2im(dev(ctx, col), [w, h], ker, stride, pad, dil).eval(ctx).numpy()
-    exact(y, O.col2im(ht(col), [w, h], ker, stride, pad, dil).numpy(), "vs oracle")
+    if dil[0] == dil[1]:
+        exact(y, O.col2im(ht(col), [w, h], ker, stride, pad, dil).numpy(), "vs oracle")
+    else:
+        with pytest.raises(RuntimeError, match="or_col2im"):
+            O.col2im(ht(col), [w, h], ker, stride, pad, dil)
+        # every pixel is the float64 sum of the entries im2col's index map sends to it (an explicit scatter of indices)
+        idx = np.arange(n * h * w * c, dtype=np.float64).reshape(n, h, w, c) + 1.0  # im2col of pixel numbers; 0 marks padding
+        src = O.im2col(ht(idx.astype(np.float32)), ker, stride, pad, dil).numpy().astype(np.int64).ravel()
+        want = np.zeros(n * h * w * c + 1)
+        np.add.at(want, src, col.astype(np.float64).ravel())
+        close(y, want[1:].reshape(n, h, w, c), 1e-5, "col2im vs the scatter of im2col's index map")
     # adjoint identity: <im2col(x), col> == <x, col2im(col)>
     x = rng.standard_normal((n, h, w, c)).astype(np.float32)
     xc = V.im2col(dev(ctx, x), ker, stride, pad, dil).eval(ctx).numpy()

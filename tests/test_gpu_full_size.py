@@ -15,7 +15,7 @@ from sage_amd.bert import BertConfig, BertLayer
 from sage_amd.layers import load_params
 from sage_amd.resnet import ResNet, ResNetConfig
 from tests.test_gpu_models import bert_layer_params, layer_param_list, resnet_arrays
-from tests.util import REL_GEMM, REL_MAP, close
+from tests.util import REL_GEMM, REL_MAP, close, exact
 
 pytestmark = pytest.mark.gpu
 
@@ -283,3 +283,58 @@ def test_streamed_maps_at_full_size_are_exact(ctx):
     e = (dev(ctx, lg) - dev(ctx, c)).exp().eval(ctx).numpy()
     close(e[:64], O.unary("exp", O.binary("sub", ht(lg[:64]), ht(c[:64]).expand([64, 1024]))).numpy(), REL_MAP, "rows vs oracle")
     assert np.all(e <= 1.0) and np.all(e.max(1) == 1.0)
+
+
+def test_config5_bert_b64_s512_under_a_memory_cap():
+    """Program::exec's memory behaviour (session.rs:259-330) on the model of configuration 5 (12 layers, b64 x s512, vocab
+    30522) in contexts whose capacity is below what an uncapped evaluation holds at its peak.
+
+    (1) The forward pass alone: intermediates die with their last consumer, so the activation peak is one operator's
+    working set (the second FFN product reads [32768,3072] and the [32768,768] residual and writes [32768,768]: 0.6 GB).
+    Under 0.9 of the peak it evicts retained tensors and recomputes them; under 0.8 that one operator's own operands no
+    longer fit and the evaluation fails with OutOfMemory, as the reference's would (it can only evict what the running
+    operator does not use, session.rs:294-325).
+    (2) The same model with every encoder layer's output kept alive by a late consumer (what a backward pass does to the
+    activations, the case the reference's eviction is for): capacity = parameters + 0.6 x the uncapped activation peak.
+    Every result is bit-identical to the uncapped one and the allocator never exceeds the capacity."""
+    import bench
+    from sage_amd import var as V
+
+    def run(capacity, retain):
+        c = S.Context(0, capacity=capacity) if capacity else S.Context(0)
+        try:
+            d = bench.build_bert(c, "config", 64, 512, 12, np.random.default_rng(5), detail=True)
+            model = d["model"]
+            if not retain:
+                targets = [d["logits"]]
+            else:
+                ids, mask, seg = (S.Var.new(S.Tensor.from_numpy(c, d[k])) for k in ("ids", "mask", "segment_ids"))
+                h = model.embedding.pass_(ids, c, seg)
+                outs = []
+                for layer in model.layers:
+                    h = layer.pass_(h, mask)
+                    outs.append(h)
+                # every layer's output is read once more, one at a time, after the last layer has run: the mean over its tokens
+                late = [o.mean(1, False) for o in outs]
+                targets = [model.classify(outs[-1])] + late
+            ev = V._Evaluator(c, targets)
+            out = np.concatenate([ev.get(t).numpy().ravel() for t in targets])
+            return out, ev.evictions, c.mem_stats(), sum(a.nbytes for a in d["arrays"])
+        finally:
+            c.close()
+
+    for retain in (False, True):
+        say("C5 under a cap, layer outputs retained:", retain)
+        want, ev0, st0, params_bytes = run(0, retain)
+        assert ev0 == 0 and np.all(np.isfinite(want))
+        act_peak = st0["peak"] - params_bytes
+        say("uncapped activation peak", act_peak, "bytes =", round(act_peak / (64 * 512 * 768 * 4), 2), "x [32768,768]")
+        frac = 0.6 if retain else 0.9
+        cap = params_bytes + int(frac * act_peak)
+        got, evictions, st, _ = run(cap, retain)
+        say("cap", frac, "evictions", evictions, "peak", st["peak"], "of", cap)
+        exact(got, want, f"capacity = parameters + {frac} x activation peak")
+        assert st["peak"] <= cap and evictions > 0
+        if not retain:
+            with pytest.raises(S.abi.OutOfMemory):
+                run(params_bytes + int(0.8 * act_peak), retain)

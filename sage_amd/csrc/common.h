@@ -52,8 +52,9 @@ struct sg_ctx {
     // Measurement switches, read from the environment ONCE, when the context is created (so that two replays of
     // one recorded program cannot round differently because the environment changed in between):
     // SAGE_GEMM_SPLITK (1..128 k ranges, 0 = the heuristic), SAGE_GEMM_TILE (0..3, -1 = the heuristic),
-    // SAGE_ATTENTION_SPLIT (0/1, -1 = the heuristic).
+    // SAGE_ATTENTION_SPLIT (0/1, -1 = the heuristic), SAGE_GEMM_DIRECT (0 = staged epilogue only).
     int force_gemm_split = 0, force_gemm_tile = -1, force_attention_split = -1;
+    int gemm_direct = 1;  // SAGE_GEMM_DIRECT=0: products always leave through the staged epilogue
     int last_gemm[7] = {0, 0, 0, 0, 0, 0, 0};  // template arguments of the most recent product kernel (BM 0: none yet)
     std::vector<void *> capture_allocs, capture_held;
     // errors

@@ -86,6 +86,8 @@ struct GemmP {
     int act, act_post;
     int vec_a, vec_b;  // 16-byte loads are legal for this operand
     int vec_c, vec_r, vec_bias;  // 16-byte accesses are legal for C rows / residual rows / the bias
+    int direct;       // epilogue without vector-ALU work is legal (set by the host, see the kernel): no activation, alpha = 1,
+                      // every C / residual offset inside a tile below 2^31 bytes, unguarded instantiation
     int k_chunk;      // split-K: workgroup z multiplies k in [z*k_chunk, min(K, (z+1)*k_chunk)); 0 = all of K
     int64_t c_sz;     // split-K: element stride between the partial results of consecutive z
     ConvG conv;       // used by the CONV instantiations only (A is then the image)
@@ -291,13 +293,48 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
+    float *C = p.C + bt0 * p.c_sb0 + bt1 * p.c_sb1 + (int64_t)blockIdx.z * p.c_sz;
+    const float *R = p.res ? p.res + bt0 * p.r_sb0 + bt1 * p.r_sb1 : nullptr;
+
+    // Direct epilogue (unguarded launches without activation or scaling): the accumulators START at bias[n] +
+    // residual[m][n] and leave, after the K loop, through buffer stores whose per-lane offset is fixed and whose
+    // per-register offset is scalar -- no vector-ALU instruction and no LDS between the last MFMA and the last
+    // store.  Vector-ALU work takes its cycles from the matrix pipe of the SIMD whichever wavefront issues it, so
+    // only a write-out made of memory instructions alone can overlap the K loop of the next workgroup on the
+    // compute unit (or of this workgroup's next tile).  Element r of a 32x32 accumulator block is row
+    // (r/4)*8 + (lane/32)*4 + r%4, column lane%32: a store instruction writes two full 128-byte row segments.
+    const bool direct = !GUARD && p.direct;
+    typedef unsigned int u32;
+    // (descriptors are per tile, hence uniform; the wavefront's block inside the tile is part of the per-lane offset)
+    const uint32_t c_lane = ((uint32_t)(wm * WM + (lane >> 5) * 4) * (uint32_t)p.c_sm + (uint32_t)(wn * WN + (lane & 31))) * 4u;
+    const uint32_t r_lane = ((uint32_t)(wm * WM + (lane >> 5) * 4) * (uint32_t)p.r_sm + (uint32_t)(wn * WN + (lane & 31))) * 4u;
+    const __amdgpu_buffer_rsrc_t c_blk = __builtin_amdgcn_make_buffer_rsrc(C + (int64_t)m0 * p.c_sm + n0, 0, -1, 0x00020000);
+
     floatx16 acc[TM][TN];
+    if (direct && (p.bias || R)) {
+        const __amdgpu_buffer_rsrc_t r_blk = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float *>(R ? R + (int64_t)m0 * p.r_sm + n0 : p.A), 0, -1, 0x00020000);
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+        for (int j = 0; j < TN; ++j) {
+            const float bj = p.bias ? p.bias[n0 + wn * WN + j * 32 + (lane & 31)] : 0.0f;
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+                for (int r = 0; r < 16; ++r) {
+                    float v = 0.0f;
+                    if (R) v = __builtin_bit_cast(float, (u32)__builtin_amdgcn_raw_buffer_load_b32(
+                                   r_blk, r_lane, ((uint32_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * (uint32_t)p.r_sm + (uint32_t)(j * 32)) * 4u, 0));
+                    acc[i][j][r] = v + bj;
+                }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    }
 
     // Two register sets for the global fetch: slab s travels through set s&1.
     f32x4 ra0[TA::NV], rb0[TB::NV], ra1[TA::NV], rb1[TB::NV];
@@ -531,9 +568,25 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     // The bias and residual values of a block are requested one block ahead (the first ones before
     // the barrier), so the rolled loop never waits a full memory round trip per row group; inside
     // the loop the four row groups' residuals sit in a small shift register to keep indices static.
+    if (direct) {
+        // (the row stride is made opaque here so that the scalar offsets below are formed now, one multiply each,
+        // instead of being hoisted above the K loop and held in registers through it)
+        uint32_t c_row = (uint32_t)p.c_sm * 4u;
+        asm volatile("" : "+s"(c_row));
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float v = acc[i][j][r];  // (a copy: bit-casting the vector element in place reads element 0)
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(u32, v), c_blk, c_lane,
+                                                          (uint32_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * c_row + (uint32_t)(j * 128), 0);
+                }
+        __syncthreads();  // every wavefront has read its last operands: the next tile may overwrite the LDS buffers
+        continue;
+    }
     float *stage = lds_raw + wave * STAGE;
-    float *C = p.C + bt0 * p.c_sb0 + bt1 * p.c_sb1 + (int64_t)blockIdx.z * p.c_sz;
-    const float *R = p.res ? p.res + bt0 * p.r_sb0 + bt1 * p.r_sb1 : nullptr;
     const int st_w = (khalf * 4) * STAGE_LD + (lane & 31);        // + ((r/4)*8 + r%4) * STAGE_LD
     const int rd_row = lane >> 3, rd_col = (lane & 7) * 4;          // + 8q rows
     auto request = [&](int blk, f32x4(&res)[4], f32x4 &bias) {
@@ -679,6 +732,54 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float *__restr
     }
 }
 
+// Products with at most 16 output columns (a classifier head: 128 x 512 x 10, 64 x 768 x 2): an MFMA tile would be
+// nearly empty and K would have to be split over workgroups and summed by a second launch to occupy more than two
+// compute units.  Here one wavefront owns one output row: its lanes walk k in steps of 64 (A[m, k] is one
+// coalesced request per step, the N values of B's row k sit side by side), every lane keeps N partial sums, and
+// the wavefront adds them up with xor-shuffles at the end.  The order of the additions is fixed (lane l sums
+// k = l, l + 64, ...; then a butterfly over the lanes): the same call gives the same bits.
+template <int NMAX>
+__global__ void __launch_bounds__(256) gemm_skinny_kernel(const GemmP p) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int m = blockIdx.x * 4 + wave;
+    if (m >= p.M) return;
+    float acc[NMAX];
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n) acc[n] = 0.0f;
+    const float *a = p.A + (int64_t)m * p.a_sm;
+    for (int k0 = 0; k0 < p.K; k0 += 256) {  // four requests per operand in flight
+        float av[4], bv[4][NMAX];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int k = k0 + u * 64 + lane;
+            av[u] = k < p.K ? a[(int64_t)k * p.a_sk] : 0.0f;
+#pragma unroll
+            for (int n = 0; n < NMAX; ++n) bv[u][n] = (k < p.K && n < p.N) ? p.B[(int64_t)k * p.b_sk + (int64_t)n * p.b_sn] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int n = 0; n < NMAX; ++n) acc[n] = __builtin_fmaf(av[u], bv[u][n], acc[n]);
+    }
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n)
+#pragma unroll
+        for (int s = 32; s >= 1; s >>= 1) acc[n] += __shfl_xor(acc[n], s, 64);
+    // lane n finishes column n
+    float v = 0.0f;
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n)
+        if (lane == n) v = acc[n];
+    if (lane < p.N) {
+        if (p.alpha != 1.0f) v *= p.alpha;
+        if (p.bias) v += p.bias[lane];
+        v = apply_act(v, p.act);
+        if (p.res) v += p.res[(int64_t)m * p.r_sm + lane];
+        v = apply_act(v, p.act_post);
+        p.C[(int64_t)m * p.c_sm + lane] = v;
+    }
+}
+
 template <int BM, int BN, int WAVES_M, bool GUARD>
 void launch_layouts(sg_ctx *ctx, const GemmP &p, dim3 grid, bool a_kc, bool b_nc) {
     dim3 block(NTHREADS);
@@ -693,6 +794,15 @@ void launch_layouts(sg_ctx *ctx, const GemmP &p, dim3 grid, bool a_kc, bool b_nc
     else if (a_kc && !b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, false, GUARD>), grid, block, 0, ctx->stream, p);
     else if (!a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, true, GUARD>), grid, block, 0, ctx->stream, p);
     else hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, false, GUARD>), grid, block, 0, ctx->stream, p);
+}
+
+// The epilogue made of buffer stores alone (see the kernel): no activation, no scaling, and every offset inside a
+// wavefront's block of C / of the residual below 2^31 bytes.  SAGE_GEMM_DIRECT=0 (read when the context is created)
+// switches it off for measurements.
+void set_direct(const sg_ctx *ctx, GemmP &p, int bm) {
+    const int64_t reach_c = (int64_t)bm * p.c_sm * 4, reach_r = p.res ? (int64_t)bm * p.r_sm * 4 : 0;
+    p.direct = ctx->gemm_direct && p.act == SG_ACT_NONE && p.act_post == SG_ACT_NONE && p.alpha == 1.0f && p.c_sm >= 0 && p.r_sm >= 0 &&
+               reach_c < (1ll << 31) && reach_r < (1ll << 31);
 }
 
 // GUARD = false needs every tile to lie fully inside the matrices and 16-byte loads to be legal.
@@ -777,6 +887,7 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noal
         const int rc_ws = workspace(ctx, (int64_t)nsplit * slice, noalloc, &ws);
         if (rc_ws != SG_OK) return rc_ws;
         GemmP q = partial_pass(p, (float *)ws, slice, k_chunk);
+        set_direct(ctx, q, BM);
         dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch, (unsigned)nsplit);
         if (needs_guard(q, BM, BN, a_kc, b_nc)) launch_layouts<BM, BN, WAVES_M, true>(ctx, q, grid, a_kc, b_nc);
         else launch_layouts<BM, BN, WAVES_M, false>(ctx, q, grid, a_kc, b_nc);
@@ -791,6 +902,7 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noal
     // walking the tiles; a batched product keeps one workgroup per tile and batch entry
     const int64_t ntiles = (int64_t)p.tiles_m * p.tiles_n, resident = 3 * (int64_t)ctx->num_cus;
     dim3 grid((unsigned)(batch == 1 && ntiles > resident ? resident : ntiles), (unsigned)batch);
+    set_direct(ctx, p, BM);
     if (needs_guard(p, BM, BN, a_kc, b_nc)) launch_layouts<BM, BN, WAVES_M, true>(ctx, p, grid, a_kc, b_nc);
     else launch_layouts<BM, BN, WAVES_M, false>(ctx, p, grid, a_kc, b_nc);
     SG_CHECK_LAUNCH(ctx, "gemm");
@@ -834,6 +946,15 @@ void launch_splitk_reduce(sg_ctx *ctx, const GemmP &p, const float *ws, int nspl
 }
 
 int launch_gemm(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noalloc) {
+    if (batch == 1 && p.conv.ohw == 0 && p.N <= 16 && ctx->force_gemm_tile < 0 && ctx->force_gemm_split == 0) {
+        dim3 grid((unsigned)((p.M + 3) / 4));
+        const int inst[7] = {-1, p.N <= 4 ? 4 : 16, 0, 0, 0, 0, 0};  // sg_gemm_last_kernel_name: gemm_skinny_kernel<NMAX>
+        for (int i = 0; i < 7; ++i) ctx->last_gemm[i] = inst[i];
+        if (p.N <= 4) hipLaunchKernelGGL((gemm_skinny_kernel<4>), grid, dim3(256), 0, ctx->stream, p);
+        else hipLaunchKernelGGL((gemm_skinny_kernel<16>), grid, dim3(256), 0, ctx->stream, p);
+        SG_CHECK_LAUNCH(ctx, "gemm (skinny)");
+        return SG_OK;
+    }
     switch (choose_tile(ctx, p.M, p.N, p.K, batch)) {
     case 0: return launch_cfg<128, 128, 2>(ctx, p, batch, a_kc, b_nc, noalloc);
     case 1: return launch_cfg<128, 96, 4>(ctx, p, batch, a_kc, b_nc, noalloc);
@@ -933,6 +1054,10 @@ extern "C" int sg_gemm_last_kernel_name(sg_ctx *ctx, char *buf, uint64_t cap) {
     if (!ctx || !buf || cap < 8) return SG_ERR_ARG;
     const int *t = ctx->last_gemm;
     if (t[0] == 0) return sg_fail(ctx, SG_ERR_ARG, "sg_gemm_last_kernel_name: no product has been launched on this context");
+    if (t[0] < 0) {
+        snprintf(buf, cap, "gemm_skinny_kernel<%d>", t[1]);
+        return SG_OK;
+    }
     snprintf(buf, cap, "gemm_mfma_kernel<%d, %d, %d, %s, %s, %s, %s>", t[0], t[1], t[2], t[3] ? "true" : "false", t[4] ? "true" : "false",
              t[5] ? "true" : "false", t[6] ? "true" : "false");
     return SG_OK;
@@ -992,28 +1117,59 @@ extern "C" int sg_conv2d(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *filte
     const int64_t want[4] = {N, OH, OW, OC};
     for (int a = 0; a < 4; ++a)
         if (out->extents[a] != want[a]) return sg_fail(ctx, SG_ERR_SHAPE, "sg_conv2d: out extent[%d] = %lld, expected %lld", a, (long long)out->extents[a], (long long)want[a]);
-    const int64_t M = N * OH * OW, K = KH * KW * Cc;
+    // Taps that lie in the padding for EVERY output pixel multiply zeros (a 3x3 window with padding 1 over a 1x1 image has
+    // one tap inside the image, over a 2-pixel-high image with stride 2 two of its three rows).  When the taps some
+    // pixel can reach form a block of the filter that is contiguous in memory (one row of taps, or whole rows), the
+    // product runs over that block alone: a smaller kernel window with the padding reduced accordingly.  The terms
+    // left out are exact zeros, so the sum keeps its value; K, and with it the split over workgroups, shrinks.
+    int64_t ky0 = 0, ky1 = KH - 1, kx0 = 0, kx1 = KW - 1;
+    int64_t ph = pad[1], pw = pad[0];
+    {
+        auto reach = [](int64_t k, int64_t n_out, int64_t s, int64_t p, int64_t d, int64_t extent) {  // some output pixel reads the image through tap k
+            for (int64_t o = 0; o < n_out; ++o) {
+                const int64_t i = o * s - p + k * d;
+                if (i >= 0 && i < extent) return true;
+                if (i >= extent) break;
+            }
+            return false;
+        };
+        int64_t a = 0, b = KH - 1, c = 0, e = KW - 1;
+        while (a < b && !reach(a, OH, stride[1], pad[1], dil[1], H)) ++a;
+        while (b > a && !reach(b, OH, stride[1], pad[1], dil[1], H)) --b;
+        while (c < e && !reach(c, OW, stride[0], pad[0], dil[0], W)) ++c;
+        while (e > c && !reach(e, OW, stride[0], pad[0], dil[0], W)) --e;
+        const bool smaller = a > 0 || b < KH - 1 || c > 0 || e < KW - 1;
+        const bool contiguous = a == b || (c == 0 && e == KW - 1);
+        if (smaller && contiguous && pad[1] - a * dil[1] >= 0 && pad[0] - c * dil[0] >= 0 && dil[0] > 0 && dil[1] > 0) {
+            ky0 = a; ky1 = b; kx0 = c; kx1 = e;
+            ph = pad[1] - a * dil[1];
+            pw = pad[0] - c * dil[0];
+        }
+    }
+    const int64_t KHe = ky1 - ky0 + 1, KWe = kx1 - kx0 + 1;  // the window the product walks
+    const int64_t M = N * OH * OW, K = KHe * KWe * Cc;
     if (M >= (1ll << 31) || K >= (1ll << 31)) return sg_fail(ctx, SG_ERR_SHAPE, "sg_conv2d: more than 2^31-1 output pixels or filter taps");
     ConvG g{};
-    g.H = (int)H; g.W = (int)W; g.C = (int)Cc; g.OW = (int)OW; g.KW = (int)KW; g.ohw = (int)(OH * OW);
-    g.sw = stride[0]; g.sh = stride[1]; g.pw = pad[0]; g.ph = pad[1]; g.dw = dil[0]; g.dh = dil[1];
+    g.H = (int)H; g.W = (int)W; g.C = (int)Cc; g.OW = (int)OW; g.KW = (int)KWe; g.ohw = (int)(OH * OW);
+    g.sw = stride[0]; g.sh = stride[1]; g.pw = (int)pw; g.ph = (int)ph; g.dw = dil[0]; g.dh = dil[1];
     g.d_ohw = sg_make_fastdiv((uint32_t)g.ohw); g.d_ow = sg_make_fastdiv((uint32_t)OW);
-    g.d_c = sg_make_fastdiv((uint32_t)Cc); g.d_kw = sg_make_fastdiv((uint32_t)KW);
+    g.d_c = sg_make_fastdiv((uint32_t)Cc); g.d_kw = sg_make_fastdiv((uint32_t)KWe);
     const float *img = (const float *)x->base + x->offset;
     g.vec = Cc % 4 == 0 && ptr_aligned16(img);
-    g.KH = (int)KH;
-    const int64_t img_bytes = N * H * W * Cc * 4, lead_bytes = ((int64_t)pad[1] * W + pad[0]) * Cc * 4;
+    g.KH = (int)KHe;
+    const int64_t img_bytes = N * H * W * Cc * 4, lead_bytes = (ph * W + pw) * Cc * 4;
     // The unguarded loads send an outside tap to lane offset 2^31 and rely on the descriptor's range check, which
     // compares against (range - scalar offset): that difference must not wrap, so the largest scalar offset of
     // the loop (last tap's displacement + the last 16-channel slab, + the 64 bytes it reads) has to lie inside
     // the range; a dilation or padding larger than the image (N = 1) can exceed it and takes the guarded loads.
-    const int64_t max_slab_off = (((KH - 1) * (int64_t)dil[1] * W + (KW - 1) * (int64_t)dil[0]) * Cc + (Cc >= 16 ? Cc - 16 : 0)) * 4 + 64;
-    g.fast = Cc % 16 == 0 && ptr_aligned16(img) && KH * KW <= 64 && img_bytes + lead_bytes < (1ll << 31) &&
+    const int64_t max_slab_off = (((KHe - 1) * (int64_t)dil[1] * W + (KWe - 1) * (int64_t)dil[0]) * Cc + (Cc >= 16 ? Cc - 16 : 0)) * 4 + 64;
+    g.fast = Cc % 16 == 0 && ptr_aligned16(img) && KHe * KWe <= 64 && img_bytes + lead_bytes < (1ll << 31) &&
              max_slab_off <= img_bytes + lead_bytes;
     g.img_bytes = g.fast ? (uint32_t)img_bytes : 0u;
     // A = the virtual [M, K] column matrix (row stride K, never dereferenced through it), B = filter as [K, OC], C = out as [M, OC]
     Mat ma{img, 0, 0, K, 1};
-    Mat mb{(const float *)filter->base + filter->offset, 0, 0, OC, 1};
+    // B = the filter rows of the taps walked: [ky0..ky1] x [kx0..kx1] x C, contiguous by the test above
+    Mat mb{(const float *)filter->base + filter->offset + (ky0 * KW + kx0) * Cc * OC, 0, 0, OC, 1};
     Mat mc{(const float *)out->base + out->offset, 0, 0, OC, 1};
     return run(ctx, (int)M, (int)OC, (int)K, 1, 1, ma, mb, mc, epi, false, &g);
 }

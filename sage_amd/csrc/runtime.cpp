@@ -76,6 +76,7 @@ int sg_ctx_create(int device_idx, uint64_t capacity_bytes, sg_ctx **out) {
     if (const char *e = getenv("SAGE_GEMM_TILE"))
         if (e[0] >= '0' && e[0] <= '3' && e[1] == 0) ctx->force_gemm_tile = e[0] - '0';
     if (const char *e = getenv("SAGE_ATTENTION_SPLIT")) ctx->force_attention_split = atoi(e) != 0;
+    if (const char *e = getenv("SAGE_GEMM_DIRECT")) ctx->gemm_direct = atoi(e) != 0;
     if (sg_gemm_device_setup(ctx) != SG_OK) {
         (void)hipStreamDestroy(ctx->stream);
         delete ctx;

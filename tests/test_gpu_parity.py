@@ -446,6 +446,29 @@ def test_gemm_random_shapes_and_layouts(ctx):
         close(out, yo.numpy(), REL_GEMM, f"case {case} vs oracle")
 
 
+@pytest.mark.parametrize("m,k,n", [(128, 512, 10), (64, 768, 2), (1, 1, 1), (7, 1000, 16), (300, 65, 3), (5, 257, 13)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_gemm_skinny_outputs(ctx, m, k, n, ta, tb):
+    """Products with at most 16 output columns (classifier heads) run one wavefront per output row instead of MFMA
+    tiles + split-K: all four transpose modes, with bias / ReLU / residual, against float64 and the oracle; the sum
+    order is fixed, so the same call gives the same bits."""
+    say("gemm skinny", (m, k, n), ta, tb)
+    rng = np.random.default_rng(m * 3 + k + n)
+    a = rng.uniform(-1, 1, (k, m) if ta else (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (n, k) if tb else (k, n)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (n,)).astype(np.float32)
+    res = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    ref64 = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+    n0 = ctx.launches
+    y = V.gemm(dev(ctx, a), dev(ctx, b), ta, tb).eval(ctx).numpy()
+    assert ctx.launches - n0 == 1
+    close(y, ref64, REL_GEMM, "gemm vs float64")
+    close(y, O.gemm(ht(a), ht(b), ta, tb).numpy(), REL_GEMM, "gemm vs oracle")
+    y2 = (nn.relu(V.gemm(dev(ctx, a), dev(ctx, b), ta, tb) + dev(ctx, bias)) + dev(ctx, res)).eval(ctx).numpy()
+    close(y2, np.maximum(ref64 + bias, 0) + res, REL_GEMM, "relu(gemm + bias) + residual vs float64")
+    exact(y, V.gemm(dev(ctx, a), dev(ctx, b), ta, tb).eval(ctx).numpy(), "same call, same bits")
+
+
 def test_gemm_batched_split_k(ctx_under):
     say("gemm_batched split-K")
     ctx = ctx_under(SAGE_GEMM_SPLITK="4")
@@ -674,6 +697,13 @@ CONV_CASES = [
     # dilation and padding larger than the image, one image: exactly tiled (M = 64, K = 288, C % 16 == 0), but the last taps'
     # displacement lies beyond the image plus its lead, so the host must choose the guarded loads
     (1, 8, 8, 32, 3, 3, 64, [1, 1], [9, 9], [9, 9]),
+    # taps that are padding for every output pixel are left out of the product when the rest of the filter is one block:
+    (8, 1, 1, 32, 3, 3, 64, [1, 1], [1, 1], [1, 1]),      # 1x1 image, 3x3 window: the centre tap alone (K 288 -> 32)
+    (64, 1, 1, 64, 3, 3, 64, [1, 1], [1, 1], [1, 1]),     # the same exactly tiled (M = 64): unguarded
+    (4, 2, 6, 16, 3, 3, 32, [1, 2], [1, 1], [1, 1]),      # 2 rows, stride 2 down: tap rows 1..2 (whole rows of the filter)
+    (2, 1, 5, 8, 3, 3, 16, [1, 1], [1, 1], [1, 1]),       # 1 row: the middle row of taps
+    (4, 2, 2, 16, 3, 3, 32, [2, 2], [1, 1], [1, 1]),      # 2x2 -> 1x1 with stride 2: taps {1,2} x {1,2}, not one block: all nine walked
+    (3, 1, 1, 5, 5, 5, 7, [1, 1], [2, 2], [1, 1]),        # 5x5 window over a 1x1 image, scalar loads
 ]
 
 
@@ -709,7 +739,7 @@ def test_conv2d_without_column_matrix(ctx, monkeypatch, case):
         if with_epilogue:
             ref = O.binary("add", O.relu(O.binary("add", yo, ht(bias))), ht(res)).numpy()
         close(y_fused, ref, REL_GEMM, "conv2d vs oracle")
-        if 512 <= kh * kw * c < 1024:
+        if 512 <= kh * kw * c < 1024 or oc <= 16:  # (a product with at most 16 columns over an existing column matrix is not an MFMA product)
             close(y_fused, y_explicit, REL_GEMM, "conv2d vs im2col + gemm")
         else:
             exact(y_fused, y_explicit, "conv2d vs im2col + gemm")
@@ -795,8 +825,12 @@ def test_last_product_kernel_name(ctx):
     a, b = dev(ctx, rng.standard_normal((256, 64)).astype(np.float32)), dev(ctx, rng.standard_normal((64, 128)).astype(np.float32))
     a.matmul(b).eval(ctx)
     assert last() == "gemm_mfma_kernel<64, 64, 2, true, true, false, false>", last()
-    dev(ctx, rng.standard_normal((70, 33)).astype(np.float32)).matmul(dev(ctx, rng.standard_normal((33, 9)).astype(np.float32))).eval(ctx)
+    dev(ctx, rng.standard_normal((70, 33)).astype(np.float32)).matmul(dev(ctx, rng.standard_normal((33, 19)).astype(np.float32))).eval(ctx)
     assert last().endswith("true, false>") and ", true, true, true, false>" in last(), last()   # guarded loads
+    dev(ctx, rng.standard_normal((70, 33)).astype(np.float32)).matmul(dev(ctx, rng.standard_normal((33, 9)).astype(np.float32))).eval(ctx)
+    assert last() == "gemm_skinny_kernel<16>", last()   # at most 16 output columns: a wavefront per output row
+    dev(ctx, rng.standard_normal((70, 33)).astype(np.float32)).matmul(dev(ctx, rng.standard_normal((33, 2)).astype(np.float32))).eval(ctx)
+    assert last() == "gemm_skinny_kernel<4>", last()
     for c, want in ((64, "gemm_mfma_kernel<64, 64, 2, true, true, false, true>"), (5, "true, true, true, true>")):
         x = S.Tensor.from_numpy(ctx, rng.standard_normal((4, 8, 8, c)).astype(np.float32))
         f = S.Tensor.from_numpy(ctx, rng.standard_normal((3, 3, c, 64)).astype(np.float32))

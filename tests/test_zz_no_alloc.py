@@ -5,6 +5,7 @@ a smaller product follows a larger one in the same array, and refuse a product w
 products do not fit.  Runs last in the suite and also passes alone in a fresh process.
 """
 import ctypes as C
+import gc
 
 import numpy as np
 import pytest
@@ -23,9 +24,16 @@ def say(*a):
 def device_free_bytes():
     """Free device memory as the HIP runtime reports it (hipMemGetInfo), asked of the runtime directly: an
     allocation made behind the context's own accounting (a stray hipMalloc in the call) would show here."""
-    hip = C.CDLL("libamdhip64.so")
+    # the runtime instance libsage_hip.so itself is linked against (a process that has imported torch holds a second,
+    # bundled HIP runtime under the same library name, which knows nothing of this library's allocations)
+    abi.lib()
+    with open("/proc/self/maps") as f:
+        paths = sorted({line.split()[-1] for line in f if "libamdhip64" in line and "/torch/" not in line})
+    assert paths, "libamdhip64 is not mapped"
+    hip = C.CDLL(paths[0])
     free, total = C.c_size_t(), C.c_size_t()
-    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    rc = hip.hipMemGetInfo(C.byref(free), C.byref(total))
+    assert rc == 0, f"hipMemGetInfo returned {rc}"
     return free.value
 
 
@@ -38,6 +46,8 @@ def product(ctx, fn, a, b, bias, res, ta=False, tb=False):
     out = S.Tensor.uninit(ctx, [m, n])
     ac, bc, oc, biasc, resc = ta_.c(), tb_.c(), out.c(), tbias.c(), tres.c()
     epi = abi.sg_gemm_epilogue(1.0, abi.ACT_RELU, abi.ACT_NONE, C.pointer(biasc), C.pointer(resc))
+    # (objects of earlier tests that die between the two readings would hand memory back to the device: collect them now)
+    gc.collect()
     ctx.sync()
     before = dict(ctx.mem_stats(), device_free=device_free_bytes())
     ctx.check(getattr(lib, fn)(ctx.handle, int(ta), int(tb), C.byref(ac), C.byref(bc), C.byref(oc), C.byref(epi)))
@@ -57,12 +67,18 @@ def test_noalloc_gemm_matches_gemm_twice_second_smaller():
             b = rng.uniform(-1, 1, (n, k) if tb else (k, n)).astype(np.float32)
             bias = rng.uniform(-1, 1, (n,)).astype(np.float32)
             res = rng.uniform(-1, 1, (m, n)).astype(np.float32)
-            want, _, _ = product(ctx, "sg_gemm", a, b, bias, res, ta, tb)
+            ctx.trim()  # so that sg_gemm's workspace has to come from the device: the control for the probe below
+            want, before0, after0 = product(ctx, "sg_gemm", a, b, bias, res, ta, tb)
             got, before, after = product(ctx, "sg_gemm_noalloc", a, b, bias, res, ta, tb)
             exact(got, want, f"sg_gemm_noalloc {m}x{k}x{n}")
             # nothing taken from (or returned to) the context's allocator, nothing new held from the device
             assert after["used"] == before["used"] and after["reserved"] == before["reserved"]
-            assert after["device_free"] == before["device_free"], "the call changed the device's free memory"
+            # ... and nothing taken from the device behind the allocator's back.  The runtime's own bookkeeping (its
+            # kernel-argument pool) may grow by a few KiB at any launch, so the bound is a size no workspace here fits in;
+            # sg_gemm, whose workspace for the first shape is megabytes, shows that the probe sees an allocation.
+            assert before["device_free"] - after["device_free"] < 128 << 10, "the call took memory from the device"
+            if (m, k, n) == (512, 2304, 256):
+                assert after0["reserved"] > before0["reserved"] and before0["device_free"] - after0["device_free"] >= 1 << 20
             ref = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
             close(got, np.maximum(ref + bias, 0) + res, REL_GEMM, "vs float64")
     finally:

@@ -24,13 +24,16 @@ def say(*a):
 def device_free_bytes():
     """Free device memory as the HIP runtime reports it (hipMemGetInfo), asked of the runtime directly: an
     allocation made behind the context's own accounting (a stray hipMalloc in the call) would show here."""
-    # the runtime instance libsage_hip.so itself is linked against (a process that has imported torch holds a second,
-    # bundled HIP runtime under the same library name, which knows nothing of this library's allocations)
+    # The runtime instance libsage_hip.so itself is bound to.  torch bundles a HIP runtime under the same library name:
+    # when torch was imported first, the loader binds this library to that copy and no other is mapped; when this
+    # library was loaded first, ROCm's own copy is mapped (and torch's, if imported later, is a second instance that
+    # knows nothing of this library's allocations).
     abi.lib()
     with open("/proc/self/maps") as f:
-        paths = sorted({line.split()[-1] for line in f if "libamdhip64" in line and "/torch/" not in line})
+        paths = sorted({line.split()[-1] for line in f if "libamdhip64" in line})
     assert paths, "libamdhip64 is not mapped"
-    hip = C.CDLL(paths[0])
+    own = [q for q in paths if "/torch/" not in q] or paths
+    hip = C.CDLL(own[0])
     free, total = C.c_size_t(), C.c_size_t()
     rc = hip.hipMemGetInfo(C.byref(free), C.byref(total))
     assert rc == 0, f"hipMemGetInfo returned {rc}"

@@ -20,6 +20,7 @@ the parity tests compare the fused results against.
 """
 import ctypes as C
 import os
+import time
 
 import numpy as np
 
@@ -990,6 +991,8 @@ class _Evaluator:
         self.release = record is None
         self.computed = set()
         self.evictions = 0
+        self.eviction_log = []  # one list of evicted tensor sizes (elements) per out-of-memory event, in eviction order
+        self.exec_time = {}
 
     # ---- helpers
     def n_users(self, v):
@@ -1005,7 +1008,11 @@ class _Evaluator:
         if t is None:
             if v.op == "data":
                 raise RuntimeError("cannot evaluate empty var")
+            t0 = time.perf_counter()
             t = getattr(self, "_ev_" + v.op)(v)
+            # Routine::exec_time (session.rs:619, 667-668): host seconds spent issuing the node (and whatever it had to
+            # evaluate first), the figure the eviction rule below reads
+            self.exec_time[id(v)] = time.perf_counter() - t0
             self.memo[id(v)] = t
             self.keep[id(v)] = v
             self.computed.add(id(v))
@@ -1041,29 +1048,23 @@ class _Evaluator:
             else:
                 stack.extend(n.inputs)
 
-    @staticmethod
-    def _recompute_cost(v):
-        """Rough time to recompute one node from its inputs (the reference measures Routine::exec_time)."""
-        n = float(v.size())
-        if v.op in GEMM_OPS:
-            a = v.inputs[0]
-            return 2.0 * n * a.extents[-1] / 1e5 + 10.0
-        if v.op in ("reduce", "reduce_arg", "softmax", "softmax_ce", "layer_norm"):
-            return float(v.inputs[0].size()) / 2e3 + 5.0
-        return n / 2e3 + 3.0
-
     def _evict(self, needed):
-        """session.rs:259-325: free at least `needed` bytes by dropping retained intermediates, cheapest
-        recompute time per byte first.  Tensors still referenced by the operator being evaluated stay
-        alive whatever is dropped here (the reference's `lock` set plays that role)."""
+        """session.rs:259-325: free at least `needed` bytes by dropping retained intermediates in the reference's
+        order: smallest (exec_time + 1.0) / (size + 1.0) first (session.rs:300-310), exec_time being the host
+        seconds measured when the node was evaluated.  (Issuing a node takes well under a second, so the rule
+        amounts to "largest tensor first", as it does in the reference; ties there fall to a hash map's iteration
+        order, here to evaluation order.)  Tensors still referenced by the operator being evaluated stay alive
+        whatever is dropped here (the reference's `lock` set plays that role)."""
         start = self.ctx.mem_stats()["used"]
         cands = [self.keep[k] for k in self.memo if k not in self.targets and k in self.keep and self.keep[k].value is None
                  and self.keep[k].op != "data"]
-        cands.sort(key=lambda n: (self._recompute_cost(n) + 1.0) / (n.size() + 1.0))
+        cands.sort(key=lambda n: (self.exec_time.get(id(n), 0.0) + 1.0) / (n.size() + 1.0))
+        self.eviction_log.append([])
         for n in cands:
             del self.memo[id(n)]
             self.computed.discard(id(n))
             self.evictions += 1
+            self.eviction_log[-1].append(n.size())
             if start - self.ctx.mem_stats()["used"] >= needed:
                 return True
         if start - self.ctx.mem_stats()["used"] >= needed:

@@ -259,6 +259,10 @@ def test_memory_capped_evaluation_evicts_and_recomputes(ctx):
             y = y + o
         ev = V._Evaluator(c, [y])
         out = ev.get(y).numpy()
+        # the reference's order (session.rs:300-310): smallest (exec_time + 1) / (size + 1) first; with issue times far
+        # below a second that is largest first
+        for sizes in ev.eviction_log:
+            assert sizes == sorted(sizes, reverse=True), sizes
         return out, ev.evictions, c.mem_stats()
 
     fresh = S.Context(0)

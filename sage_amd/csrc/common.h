@@ -119,10 +119,11 @@ int sg_validate_tensor(sg_ctx *ctx, const sg_tensor *t, const char *name);
 // gemm.hip: per-device set-up (the address of the static split-K scratch), run by sg_ctx_create.
 int sg_gemm_device_setup(sg_ctx *ctx);
 
-// A kernel that moves this many bytes streams them: past this size nothing it reads or writes is
-// found in the caches by its neighbours in the queue anyway, and non-temporal loads and stores
-// (no allocation in the L2s on the way through) sustain about a fifth more HBM bandwidth.
-// SAGE_STREAM_MIN_BYTES overrides the threshold (0 = always stream).
+// A kernel that moves at least 16 MiB streams them: a consumer's workgroups sit on any of the 8 XCDs, so what a
+// kernel leaves in one XCD's L2 serves an eighth of its readers at best, while stores that stay dirty in the L2s are
+// written back in one burst when the kernel ends; non-temporal loads and stores (no allocation in the L2s on the
+// way through) sustain about a fifth more HBM bandwidth.  SAGE_STREAM_MIN_BYTES overrides the threshold
+// (0 = always stream); BERT-base b32 x s128, whose LayerNorms move 25 MB each: 5.731 -> 5.717 ms per step.
 bool sg_streaming(int64_t bytes);
 
 // Magic-number unsigned division for n < 2^31: q = (umulhi(n, magic) + n) >> shift.

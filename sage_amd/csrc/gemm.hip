@@ -747,17 +747,18 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const GemmP p) {
 #pragma unroll
     for (int n = 0; n < NMAX; ++n) acc[n] = 0.0f;
     const float *a = p.A + (int64_t)m * p.a_sm;
-    for (int k0 = 0; k0 < p.K; k0 += 256) {  // four requests per operand in flight
-        float av[4], bv[4][NMAX];
+    constexpr int U = NMAX <= 4 ? 8 : 4;  // requests per operand in flight (more would not fit the registers at 16 columns)
+    for (int k0 = 0; k0 < p.K; k0 += 64 * U) {
+        float av[U], bv[U][NMAX];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const int k = k0 + u * 64 + lane;
             av[u] = k < p.K ? a[(int64_t)k * p.a_sk] : 0.0f;
 #pragma unroll
             for (int n = 0; n < NMAX; ++n) bv[u][n] = (k < p.K && n < p.N) ? p.B[(int64_t)k * p.b_sk + (int64_t)n * p.b_sn] : 0.0f;
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int n = 0; n < NMAX; ++n) acc[n] = __builtin_fmaf(av[u], bv[u][n], acc[n]);
     }
@@ -946,7 +947,10 @@ void launch_splitk_reduce(sg_ctx *ctx, const GemmP &p, const float *ws, int nspl
 }
 
 int launch_gemm(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noalloc) {
-    if (batch == 1 && p.conv.ohw == 0 && p.N <= 16 && ctx->force_gemm_tile < 0 && ctx->force_gemm_split == 0) {
+    // (a wavefront per row pays while the rows are few: 128 x 512 x 10 takes 7.7 us against 13.7 for tile + split-K + second pass,
+    // 64 x 768 x 2 4.5 against 13; a lane's reads of B are 4 bytes at a stride of N floats, so thousands of rows are better off
+    // in MFMA tiles: 1024 x 512 x 16 took 18 us, 32768 x 768 x 2 43 us)
+    if (batch == 1 && p.conv.ohw == 0 && p.N <= 16 && p.M <= 512 && ctx->force_gemm_tile < 0 && ctx->force_gemm_split == 0) {
         dim3 grid((unsigned)((p.M + 3) / 4));
         const int inst[7] = {-1, p.N <= 4 ? 4 : 16, 0, 0, 0, 0, 0};  // sg_gemm_last_kernel_name: gemm_skinny_kernel<NMAX>
         for (int i = 0; i < 7; ++i) ctx->last_gemm[i] = inst[i];

@@ -23,7 +23,7 @@ int sg_fail(sg_ctx *ctx, int code, const char *fmt, ...) {
 bool sg_streaming(int64_t bytes) {
     static const int64_t min_bytes = [] {
         const char *e = getenv("SAGE_STREAM_MIN_BYTES");
-        return e ? (int64_t)strtoll(e, nullptr, 10) : (int64_t)32 << 20;
+        return e ? (int64_t)strtoll(e, nullptr, 10) : (int64_t)16 << 20;
     }();
     return bytes >= min_bytes;
 }

@@ -446,11 +446,11 @@ def test_gemm_random_shapes_and_layouts(ctx):
         close(out, yo.numpy(), REL_GEMM, f"case {case} vs oracle")
 
 
-@pytest.mark.parametrize("m,k,n", [(128, 512, 10), (64, 768, 2), (1, 1, 1), (7, 1000, 16), (300, 65, 3), (5, 257, 13)])
+@pytest.mark.parametrize("m,k,n", [(128, 512, 10), (64, 768, 2), (1, 1, 1), (7, 1000, 16), (300, 65, 3), (5, 257, 13), (512, 129, 16), (513, 129, 16)])
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
 def test_gemm_skinny_outputs(ctx, m, k, n, ta, tb):
-    """Products with at most 16 output columns (classifier heads) run one wavefront per output row instead of MFMA
-    tiles + split-K: all four transpose modes, with bias / ReLU / residual, against float64 and the oracle; the sum
+    """Products with at most 16 output columns and at most 512 rows (classifier heads) run one wavefront per output row
+    instead of MFMA tiles + split-K (513 rows: tiles again): all four transpose modes, with bias / ReLU / residual, against float64 and the oracle; the sum
     order is fixed, so the same call gives the same bits."""
     say("gemm skinny", (m, k, n), ta, tb)
     rng = np.random.default_rng(m * 3 + k + n)

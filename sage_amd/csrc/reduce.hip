@@ -56,6 +56,30 @@ template <int OP, class T> __device__ __forceinline__ T wave_reduce(T v) {
     return v;
 }
 
+// The same over the 64 lanes for fp32 with data-parallel-primitive moves instead of LDS permutes: a butterfly step
+// through ds_bpermute costs an address computation and an LDS round trip (six of them in a row, twice for a
+// LayerNorm row, while the row's registers wait), a DPP move is one vector instruction.  Quad permutes give
+// every lane its quad's total, two row shifts leave the row's total in lanes 12..15, two row broadcasts carry it
+// across the four rows into lane 63, which is read back as a scalar.  Lanes a move does not reach receive the
+// operator's identity.  (A fixed tree: the same input gives the same bits.)
+template <int OP> __device__ __forceinline__ float wave_reduce_dpp(float v) {
+    const int id = __builtin_bit_cast(int, identity<OP, float>());
+#define SG_DPP_STEP(CTRL, ROW_MASK) \
+    v = combine<OP, float>(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(id, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false)))
+    SG_DPP_STEP(0xb1, 0xf);   // quad_perm:[1,0,3,2]
+    SG_DPP_STEP(0x4e, 0xf);   // quad_perm:[2,3,0,1]
+    SG_DPP_STEP(0x114, 0xf);  // row_shr:4
+    SG_DPP_STEP(0x118, 0xf);  // row_shr:8
+    SG_DPP_STEP(0x142, 0xa);  // row_bcast:15 into rows 1 and 3
+    SG_DPP_STEP(0x143, 0xc);  // row_bcast:31 into rows 2 and 3
+#undef SG_DPP_STEP
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+template <> __device__ __forceinline__ float wave_reduce<OP_SUM, float>(float v) { return wave_reduce_dpp<OP_SUM>(v); }
+template <> __device__ __forceinline__ float wave_reduce<OP_MAX, float>(float v) { return wave_reduce_dpp<OP_MAX>(v); }
+template <> __device__ __forceinline__ float wave_reduce<OP_MIN, float>(float v) { return wave_reduce_dpp<OP_MIN>(v); }
+template <> __device__ __forceinline__ float wave_reduce<OP_PROD, float>(float v) { return wave_reduce_dpp<OP_PROD>(v); }
+
 struct Dims {
     int n;
     uint32_t ext[SG_MAX_RANK];
@@ -280,6 +304,7 @@ __device__ __forceinline__ void load_row(const float *p, uint32_t len, int li, R
 }
 
 template <int OP, int LPR> __device__ __forceinline__ float seg_reduce(float v) {
+    if (LPR == WAVE) return wave_reduce<OP, float>(v);
 #pragma unroll
     for (int m = LPR / 2; m >= 1; m >>= 1) v = combine<OP, float>(v, shfl_xor(v, m));
     return v;

@@ -350,6 +350,66 @@ def test_unslice_concat(ctx):
     exact(V.concat([dev(ctx, a), dev(ctx, b), cd], 1).eval(ctx).numpy(), O.concat([ht(a), ht(b), co], 1).numpy(), "concat")
 
 
+def _random_view(rng, ext):
+    """A host array and a layout operation (for view_pair) whose result has extents `ext`: the array is stored with its
+    axes permuted, with room for a slice along one axis, and with some extent-1 axes broadcast to their extent."""
+    rank = len(ext)
+    perm = [int(p) for p in rng.permutation(rank)]          # stored axis i holds logical axis perm[i]
+    stored = [ext[p] for p in perm]
+    cut = int(rng.integers(0, rank))                            # stored axis that is sliced out of a larger one
+    lo = int(rng.integers(0, 3))
+    stored[cut] += lo + int(rng.integers(0, 3))
+    bcast = [a for a in range(rank) if ext[a] > 1 and rng.uniform() < 0.2]   # logical axes stored with extent 1
+    for a in bcast:
+        if perm.index(a) != cut:
+            stored[perm.index(a)] = 1
+    inv = [perm.index(a) for a in range(rank)]
+
+    def fn(t):
+        t = t.slice(cut, lo, lo + (1 if stored[cut] == 1 else ext[perm[cut]]))
+        t = t.permute(inv)
+        return t.expand(list(ext))
+    return stored, fn
+
+
+def test_index_kernels_on_random_views(ctx):
+    """gather, scatter, unslice and concat over 30 seeded random cases of rank 1..6: operands stored permuted, as windows of
+    larger arrays and with broadcast axes, so that the host-side collapse of the index space meets merged, unmergeable and
+    vanishing axes around the gather / scatter axis.  Integer data, so every result (duplicate scatter targets included)
+    is exact against the oracle, whose index arithmetic is pinned by explicit loops on the CPU."""
+    rng = np.random.default_rng(2024)
+    for case in range(30):
+        rank = int(rng.integers(1, 7))
+        ext = [int(rng.integers(1, 6)) for _ in range(rank)]
+        axis = int(rng.integers(0, rank))
+        say("index kernels on random views", case, ext, axis)
+        # gather: x's extents >= ind's except along the axis
+        xext = [e + int(rng.integers(0, 3)) for e in ext]
+        xext[axis] = int(rng.integers(1, 7))
+        xs, xfn = _random_view(rng, xext)
+        isz, ifn = _random_view(rng, ext)
+        x = rng.integers(0, 1 << 20, xs).astype(np.uint32)
+        ind = rng.integers(0, xext[axis], isz).astype(np.uint32)
+        (xd, xo), (idd, ido) = view_pair(ctx, x, xfn), view_pair(ctx, ind, ifn)
+        exact(V.gather(xd, idd, axis).eval(ctx).numpy(), O.gather(xo, ido, axis).numpy(), f"gather case {case}")
+        # scatter: ind dense (the reference decomposes by ind's own strides), x any view with ind's extents, duplicates allowed
+        oext = [e + int(rng.integers(0, 2)) for e in ext]
+        oext[axis] = int(rng.integers(1, 5))
+        ss, sfn = _random_view(rng, ext)
+        src = rng.integers(0, 1000, ss).astype(np.uint32)
+        ind2 = rng.integers(0, oext[axis], ext).astype(np.uint32)
+        sd, so = view_pair(ctx, src, sfn)
+        exact(V.scatter(sd, dev(ctx, ind2), axis, oext).eval(ctx).numpy(), O.scatter(so, ht(ind2), axis, oext).numpy(), f"scatter case {case}")
+        # unslice and concat along the axis
+        start = int(rng.integers(0, 3))
+        end = start + ext[axis] + int(rng.integers(0, 3))
+        exact(V.unslice(sd, axis, start, end).eval(ctx).numpy(), O.unslice(so, axis, start, end).numpy(), f"unslice case {case}")
+        other = list(ext)
+        other[axis] = int(rng.integers(1, 4))
+        b = rng.integers(0, 1000, other).astype(np.uint32)
+        exact(V.concat([sd, dev(ctx, b), sd], axis).eval(ctx).numpy(), O.concat([so, ht(b), so], axis).numpy(), f"concat case {case}")
+
+
 # ----------------------------------------------------------------------------- GEMM
 @pytest.mark.parametrize("mkn", [(1, 1, 1), (7, 13, 5), (128, 128, 128), (130, 257, 70), (64, 49, 64), (256, 64, 96), (33, 300, 200), (1, 512, 10), (300, 1, 17)])
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])

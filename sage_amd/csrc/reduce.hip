@@ -493,8 +493,12 @@ __global__ void __launch_bounds__(256) softmax_ce_row_generic_kernel(const float
 // y = (x - mean) / sqrt(var + eps) * gamma + beta.  The division by sqrt(var+eps) is applied as a
 // multiplication by its reciprocal (one division per row); everything else keeps the reference's
 // operation order.
+// Streaming launches are held to five wavefronts per SIMD: with all eight resident, a quarter more rows are in flight
+// than the memory system serves at its best rate and every one of them holds its 3 KB until its statistics are complete
+// ([32768,768]: 35.3 us with eight, 34.7 with six, 34.1 with five, 34.6 with four, 38.1 with three; the other row kernels
+// lose with fewer than eight).
 template <int NCHUNK, int LPR, bool NT>
-__global__ void __launch_bounds__(256) layer_norm_row_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NT ? 5 : 8, NT ? 5 : 8))) layer_norm_row_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
                                                              const float *__restrict__ beta, float *__restrict__ y,
                                                              uint32_t n_rows, uint32_t len, uint32_t x_off, Dims xo,
                                                              uint32_t g_off, uint32_t g_stride, uint32_t b_off, uint32_t b_stride,

@@ -535,20 +535,29 @@ def main():
     ctx = S.Context(0)
     res, keep = time_model(ctx, a.workload, a.variant, a.batch, a.seq, a.layers, a.steps, a.warmup, a.graph != "off")
     headline = a.workload == "bert" and (a.batch, a.seq, a.layers, a.variant) == (32, 128, 12, "config")
+    # The headline is measured; what follows adds to the line.  A failure in one of the additions is reported in the
+    # line (`<key>_error`) instead of costing the headline its record.
+    def added(key, make):
+        try:
+            res[key] = make()
+        except Exception as e:  # noqa: BLE001
+            res[key + "_error"] = f"{type(e).__name__}: {e}"[:400]
+            print(f"bench.py: {key} failed: {e}", file=sys.stderr)
+
     if a.workload == "bert" and not a.no_hbm_kernels:
         # the other half of the metric: the fused map / reduce / row kernels against the HBM peak, each beside a
         # plain copy of the same number of bytes timed in this same run (what a launch of that size can reach)
         ctx.trim()
-        res["roofline_hbm"] = hbm_rooflines(ctx)
+        added("roofline_hbm", lambda: hbm_rooflines(ctx))
     if headline and not a.no_configs:
-        res["configs"] = other_configs(ctx, res)
+        added("configs", lambda: other_configs(ctx, res))
     if not a.no_cpu_baseline:
         if a.workload == "resnet18":
-            res["cpu_baseline"] = cpu_baseline_resnet18(keep["model"], keep["arrays"], keep["x_host"])
+            added("cpu_baseline", lambda: cpu_baseline_resnet18(keep["model"], keep["arrays"], keep["x_host"]))
         elif a.batch * a.seq <= 4096:
-            res["cpu_baseline"] = cpu_baseline_whole_model(keep["bert"], a.variant, a.layers, keep["out0"])
+            added("cpu_baseline", lambda: cpu_baseline_whole_model(keep["bert"], a.variant, a.layers, keep["out0"]))
         else:
-            res["cpu_baseline"] = cpu_baseline(a.variant, a.batch, a.seq, 6)
+            added("cpu_baseline", lambda: cpu_baseline(a.variant, a.batch, a.seq, 6))
     print(json.dumps(res))
 
 
@@ -696,7 +705,11 @@ def other_configs(ctx, headline):
                              "flops_per_launch": cfg["flops_per_step"], "achieved": roof["achieved"], "unit": "TFLOP/s", "launches_timed": 200}})
     ctx.trim()
     for workload, batch, seq, steps, warmup in (("resnet18", 128, 0, 50, 10), ("bert", 64, 512, 6, 2)):
-        r, _ = time_model(ctx, workload, "config", batch, seq, 12, steps, warmup, True)
+        try:
+            r, _ = time_model(ctx, workload, "config", batch, seq, 12, steps, warmup, True)
+        except Exception as e:  # noqa: BLE001  (the other entries stay)
+            out.append({"workload": f"{workload}_b{batch}", "error": f"{type(e).__name__}: {e}"[:400]})
+            continue
         rf = r["roofline"]
         out.append({"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "value": r["value"], "unit": r["unit"], "steps": steps,
                     "launches_per_step": r["config"]["launches_per_step"], "gemm_tflops_whole_step": r["config"]["gemm_tflops_whole_step"],

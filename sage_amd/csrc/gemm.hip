@@ -32,7 +32,11 @@
 //     of tiles, which keeps the A/B panels a tile group shares inside that XCD's L2.
 //   * The epilogue applies alpha, bias[n], activation and a residual on the way out: accumulator
 //     blocks go through a per-wavefront LDS stage and leave as 16-byte row segments, in a rolled
-//     loop that keeps the kernel's code small.
+//     loop that keeps the kernel's code small.  Unguarded launches without activation or scaling
+//     skip all of that: their accumulators start at bias + residual and leave through buffer stores
+//     alone, so nothing after the last MFMA costs the matrix pipe a cycle.
+//   * Products with at most 16 columns and a few hundred rows (classifier heads) do not use tiles
+//     at all: gemm_skinny_kernel gives every output row a wavefront.
 // Accumulation order differs from the reference's sequential k (MFMA sums pairs of k, slabs in
 // order); the difference is fp32 rounding only and is covered by the 1e-3 GEMM tolerance.
 #include "common.h"

@@ -1,11 +1,14 @@
-// Indexing kernels for gfx950: gather, scatter, unslice, concat, im2col, fill.
+// Indexing kernels for gfx950: gather, scatter, unslice, concat, im2col, col2im, pooling, fill.
 //
 // These replace the reference's generated kernels of ops/core.rs (gather core.rs:674-705, scatter
-// :784-819, unslice :591-600, concat :917-924) and ops/conv.rs (im2col conv.rs:304-349).  They are
-// pure data movement: results are bit-exact copies.  Each thread owns consecutive output elements
-// along the innermost (contiguous) output axis so stores are coalesced; coordinates come from a
-// per-thread mixed-radix decomposition instead of the reference's per-axis loop of divisions, and
-// im2col is parallel over every output element instead of looping batch*KH*KW inside a work-item.
+// :784-819, unslice :591-600, concat :917-924) and ops/conv.rs (im2col conv.rs:304-349, col2im
+// conv.rs:418-473).  They are data movement (col2im and pooling add): results are bit-exact.  Each thread
+// owns consecutive output elements along the innermost (contiguous) output axis so stores are coalesced.
+// Coordinates come from a mixed-radix decomposition of the thread's linear index, where the reference
+// divides and takes remainders per axis and element (core.rs:162-167): here the index space is collapsed
+// on the host first (axes of extent 1 vanish, neighbouring axes that every operand walks like one axis
+// merge) and what remains is decomposed with multiply-high magic numbers, so no kernel divides in
+// hardware; im2col is parallel over every output element instead of looping batch*KH*KW inside a work-item.
 #include "common.h"
 
 namespace {

@@ -25,9 +25,13 @@
 //   * On this hardware the vector ALU and the matrix pipe of a SIMD exclude each other, across
 //     wavefronts: while one wavefront issues MFMAs back to back no other wavefront of that SIMD
 //     gets a vector instruction through (LDS, memory and scalar instructions do issue), and every
-//     vector instruction costs the matrix pipe its cycles.  Hence no vector address arithmetic in
-//     the K loop, a short branch-free erf in the GELU epilogue, and workgroups that walk tiles
-//     (the loops of the workgroups on a compute unit run one after the other anyway).
+//     vector instruction costs the matrix pipe its cycles (about 17 per instruction that interrupts a
+//     run of MFMAs).  Hence no vector address arithmetic in the K loop -- global requests are buffer
+//     loads with fixed per-lane offsets, LDS reads take fixed per-lane origins plus immediates (nine
+//     address additions per two slabs, which the compiler had placed there for paired LDS reads, cost
+//     6 % of a 128x96 loop: 1640 cycles per slab against the 1536 of its 24 MFMAs, now 1539) -- a short
+//     branch-free erf in the GELU epilogue, and workgroups that walk tiles (the loops of the workgroups
+//     on a compute unit run one after the other anyway).
 //   * Workgroup ids are remapped so that the ids one XCD receives (id mod 8) cover a compact block
 //     of tiles, which keeps the A/B panels a tile group shares inside that XCD's L2.
 //   * The epilogue applies alpha, bias[n], activation and a residual on the way out: accumulator
@@ -51,7 +55,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));  // native vector: stay
 
 constexpr int BK = 16;   // k-slab
 constexpr int KPAD = 4;  // row padding of [row][k] LDS tiles (floats)
-constexpr int RPAD = 4;  // row padding of [k][row] LDS tiles (floats)
 constexpr int NTHREADS = 256;
 constexpr int NUM_XCD = 8;
 
@@ -134,13 +137,13 @@ __device__ __forceinline__ void apply_act4(f32x4 &v, int act) {
 // K_CONTIG: the operand is contiguous along k in global memory.  The tile is then kept in LDS as
 // [row][k] (row stride BK+KPAD floats) and an MFMA operand fetch is ONE 16-byte read of 4
 // consecutive k; with the padding, 8 consecutive rows cover all 32 banks.  Otherwise the operand is
-// contiguous along its rows, the tile is kept as [k][row] (row stride ROWS+RPAD) and a fetch is a
-// 4-byte read of 32 consecutive floats per half-wave.  Either way global loads and LDS stores are
-// 16 bytes wide and no transposition happens on the way.
+// contiguous along its rows, the tile is kept as [k][row] (row stride ROWS rounded up to 64 floats, see
+// fetch()) and a fetch is a 4-byte read of 32 consecutive floats per half-wave.  Either way global loads
+// and LDS stores are 16 bytes wide and no transposition happens on the way.
 template <int ROWS, bool K_CONTIG> struct Tile {
     static constexpr int TOTAL = ROWS * BK / 4;                      // float4 per slab
     static constexpr int NV = (TOTAL + NTHREADS - 1) / NTHREADS;     // float4 per thread (last may be partial)
-    static constexpr int LD = K_CONTIG ? BK + KPAD : ROWS + RPAD;
+    static constexpr int LD = K_CONTIG ? BK + KPAD : (ROWS + 63) / 64 * 64;
     static constexpr int SIZE = K_CONTIG ? ROWS * LD : BK * LD;      // floats
 
     // When the slab does not divide evenly over the threads, the surplus slots of the last round
@@ -226,15 +229,20 @@ template <int ROWS, bool K_CONTIG> struct Tile {
         *reinterpret_cast<f32x4 *>(&lds[lds_at(row, k)]) = r;
     }
 
-    // MFMA operands of one group of 4 k-steps for the 32 rows starting at `col0`: step s of group g
-    // multiplies k = 8g + 4*(lane/32) + s.
-    __device__ static __forceinline__ void fetch(const float *lds, int col, int g, int khalf, float out[4]) {
+    // MFMA operands of one group of 4 k-steps for one 32-row block: step s of group g multiplies
+    // k = 8g + 4*(lane/32) + s.  `at` is the byte offset in LDS of the lane's (row, k = 4*(lane/32)) element of the block
+    // in buffer 0 (fetch_origin(), worked out once per kernel); what a fetch adds to it is a compile-time constant, so
+    // the loop holds no address arithmetic.  Kept [k][row], a lane's four k are LD floats apart: LD is a multiple of 64
+    // floats, which lets two of them share one instruction (a pair of reads 64-dword units apart) from the same address.
+    __device__ static __forceinline__ uint32_t fetch_origin(int col, int khalf) { return (uint32_t)(K_CONTIG ? col * LD + 4 * khalf : 4 * khalf * LD + col) * 4u; }
+    __device__ static __forceinline__ void fetch(const float *lds, uint32_t at, int buf, int g, float out[4]) {
+        const char *p = reinterpret_cast<const char *>(lds) + at + (uint32_t)(buf * SIZE * 4);
         if (K_CONTIG) {
-            const f32x4 v = *reinterpret_cast<const f32x4 *>(&lds[col * LD + 8 * g + 4 * khalf]);
+            const f32x4 v = *reinterpret_cast<const f32x4 *>(p + 8 * g * 4);
             out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
         } else {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) out[s] = lds[(8 * g + 4 * khalf + s) * LD + col];
+            for (int s = 0; s < 4; ++s) out[s] = *reinterpret_cast<const float *>(p + (8 * g + s) * LD * 4);
         }
     }
 };
@@ -346,6 +354,19 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     constexpr int NRB = TM + TN;          // operand fetches (one per 32-row block) per group of k-steps
     constexpr int NMFMA = 4 * TM * TN;    // MFMAs per group
     const int a_col = wm * WM + (lane & 31), b_col = wn * WN + (lane & 31), khalf = lane >> 5;
+    // where this lane's operands of each 32-row block start in LDS (bytes from lds_raw, buffer 0); opaque to the
+    // compiler, which would otherwise fold them into fresh address registers inside the loop
+    uint32_t a_at[TM], b_at[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        a_at[i] = TA::fetch_origin(a_col + i * 32, khalf);
+        asm volatile("" : "+v"(a_at[i]));
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        b_at[j] = (uint32_t)(2 * TA::SIZE * 4) + TB::fetch_origin(b_col + j * 32, khalf);
+        asm volatile("" : "+v"(b_at[j]));
+    }
     float a0[TM][4], b0[TN][4], a1[TM][4], b1[TN][4];
 
     // unguarded path: per-lane byte offsets of this thread's items inside a slab, and the tile bases
@@ -469,10 +490,10 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     do {                                                                                       \
         if ((e) < TM) {                                                                        \
             const int ia = (e) < TM ? (e) : 0;                                             \
-            TA::fetch(lds_a[BUF], a_col + ia * 32, G, khalf, AR[ia]);                          \
+            TA::fetch(lds_raw, a_at[ia], BUF, G, AR[ia]);                                      \
         } else {                                                                               \
             const int ib = (e) >= TM ? (e) - TM : 0;                                       \
-            TB::fetch(lds_b[BUF], b_col + ib * 32, G, khalf, BR[ib]);                          \
+            TB::fetch(lds_raw, b_at[ib], BUF, G, BR[ib]);                                      \
         }                                                                                      \
     } while (0)
 #define SG_MFMA_OP(ACC, A_, B_) ACC = __builtin_amdgcn_mfma_f32_32x32x2f32(A_, B_, ACC, 0, 0, 0)
@@ -905,7 +926,8 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noal
     }
     // one workgroup per tile while they all fit at once (three per compute unit), else that many workgroups
     // walking the tiles; a batched product keeps one workgroup per tile and batch entry
-    const int64_t ntiles = (int64_t)p.tiles_m * p.tiles_n, resident = 3 * (int64_t)ctx->num_cus;
+    static const int res_per_cu = getenv("SAGE_GEMM_RESIDENT") ? atoi(getenv("SAGE_GEMM_RESIDENT")) : 3;  // EXPERIMENT
+    const int64_t ntiles = (int64_t)p.tiles_m * p.tiles_n, resident = res_per_cu * (int64_t)ctx->num_cus;
     dim3 grid((unsigned)(batch == 1 && ntiles > resident ? resident : ntiles), (unsigned)batch);
     set_direct(ctx, p, BM);
     if (needs_guard(p, BM, BN, a_kc, b_nc)) launch_layouts<BM, BN, WAVES_M, true>(ctx, p, grid, a_kc, b_nc);

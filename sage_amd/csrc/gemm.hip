@@ -322,31 +322,11 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     const uint32_t r_lane = ((uint32_t)(wm * WM + (lane >> 5) * 4) * (uint32_t)p.r_sm + (uint32_t)(wn * WN + (lane & 31))) * 4u;
     const __amdgpu_buffer_rsrc_t c_blk = __builtin_amdgcn_make_buffer_rsrc(C + (int64_t)m0 * p.c_sm + n0, 0, -1, 0x00020000);
 
+    // The requests are ordered so that nothing waits for memory twice: further down, the first two operand slabs,
+    // then the residual straight into the accumulator registers, then the bias (a handful of values), which is added
+    // once the first operands sit in LDS, right in front of the loop.
     floatx16 acc[TM][TN];
-    if (direct && (p.bias || R)) {
-        const __amdgpu_buffer_rsrc_t r_blk = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<float *>(R ? R + (int64_t)m0 * p.r_sm + n0 : p.A), 0, -1, 0x00020000);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const float bj = p.bias ? p.bias[n0 + wn * WN + j * 32 + (lane & 31)] : 0.0f;
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    float v = 0.0f;
-                    if (R) v = __builtin_bit_cast(float, (u32)__builtin_amdgcn_raw_buffer_load_b32(
-                                   r_blk, r_lane, ((uint32_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * (uint32_t)p.r_sm + (uint32_t)(j * 32)) * 4u, 0));
-                    acc[i][j][r] = v + bj;
-                }
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-    }
+    float bias_j[TN];
 
     // Two register sets for the global fetch: slab s travels through set s&1.
     f32x4 ra0[TA::NV], rb0[TB::NV], ra1[TA::NV], rb1[TB::NV];
@@ -566,6 +546,30 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     for (int e = 0; e < NWR; ++e) SG_ITEM_LOAD(e, ra0, rb0, 0);
 #pragma unroll
     for (int e = 0; e < NWR; ++e) SG_ITEM_LOAD(e, ra1, rb1, BK);
+    __builtin_amdgcn_sched_barrier(0);  // (the operand requests above leave before the residual's)
+    if (direct && R) {
+        const __amdgpu_buffer_rsrc_t r_blk = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(R + (int64_t)m0 * p.r_sm + n0), 0, -1, 0x00020000);
+        uint32_t r_row = (uint32_t)p.r_sm * 4u;
+        asm volatile("" : "+s"(r_row));  // (scalar offsets formed here, one multiply each, not held in registers from further up)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[i][j][r] = __builtin_bit_cast(float, (u32)__builtin_amdgcn_raw_buffer_load_b32(
+                        r_blk, r_lane, (uint32_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * r_row + (uint32_t)(j * 128), 0));
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bias_j[j] = direct && p.bias ? p.bias[n0 + wn * WN + j * 32 + (lane & 31)] : 0.0f;
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int e = 0; e < NWR; ++e) SG_ITEM_STORE(e, ra0, rb0, 0);
 #pragma unroll
@@ -573,6 +577,14 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     __syncthreads();
 #pragma unroll
     for (int e = 0; e < NRB; ++e) SG_ITEM_FETCH(e, 0, 0, a0, b0);
+    if (direct && p.bias) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] += bias_j[j];
+    }
     for (int kt = 0; kt < nk; kt += 2) {
         SG_SLAB_BODY(kt, ra1, rb1);
         SG_SLAB_BODY(kt + 1, ra0, rb0);

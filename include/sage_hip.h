@@ -75,6 +75,21 @@ typedef struct sg_ctx sg_ctx;
  * the bytes handed out by sg_alloc (Allocator::new capacity, memory.rs:173-180); 0 = no cap beyond
  * the device.  The reference default is SG_REFERENCE_CAPACITY_BYTES. */
 int sg_ctx_create(int device_idx, uint64_t capacity_bytes, sg_ctx **out);
+/* The same with the allocator's two switches, Allocator::new(capacity, use_cache, use_sub_buffer) (memory.rs:64-69,
+ * 224-236).  use_cache = 0 is sg_ctx_create (what the reference's Context builds, context.rs:49).  use_cache = 1
+ * takes memory from the device in chunks and serves requests from them, Pool::alloc's caching branch
+ * (memory.rs:262-352, 364-475): requests below 1 MiB from 2 MiB chunks, larger ones from 20 MiB chunks, requests
+ * of 10 MiB and more from chunks of their own size rounded up to 2 MiB (allocation_size, memory.rs:257-265); the
+ * smallest free block that fits and is not wastefully large (a request below 40 MiB never takes a block of 40 MiB
+ * or more, a larger one never a block 20 MiB beyond its size), split when the rest is worth keeping (>= 512 B
+ * behind a request up to 1 MiB, > 1 MiB behind one below 40 MiB; use_sub_buffer = 0: never split), neighbours of
+ * one chunk merged again when freed; when nothing fits: whole free chunks older than the average age are returned
+ * to the device once 80 % of the capacity is in use, a new chunk is taken, and if the capacity forbids that the
+ * largest whole free chunks of the large class are returned first (then, beyond the reference, those of the small
+ * class).  Sizes are rounded up to 256 B so that every block keeps the
+ * alignment of a device allocation.  sg_mem_stats then reports used = bytes of the blocks handed out, reserved =
+ * bytes of the chunks held (the figure the capacity bounds, Pool::check_space), peak = the most ever held. */
+int sg_ctx_create_pooled(int device_idx, uint64_t capacity_bytes, int use_cache, int use_sub_buffer, sg_ctx **out);
 int sg_ctx_destroy(sg_ctx *ctx);
 
 /* Context::alloc -> Pool::alloc -> Device::alloc_buffer (context.rs:119-137, memory.rs:353-362,

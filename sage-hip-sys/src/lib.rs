@@ -176,6 +176,7 @@ pub struct sg_graph {
 extern "C" {
     // ---- context, memory, transfers
     pub fn sg_ctx_create(device_idx: c_int, capacity_bytes: u64, out: *mut *mut sg_ctx) -> c_int;
+    pub fn sg_ctx_create_pooled(device_idx: c_int, capacity_bytes: u64, use_cache: c_int, use_sub_buffer: c_int, out: *mut *mut sg_ctx) -> c_int;
     pub fn sg_ctx_destroy(ctx: *mut sg_ctx) -> c_int;
     pub fn sg_alloc(ctx: *mut sg_ctx, nbytes: u64, dptr: *mut *mut c_void) -> c_int;
     pub fn sg_free(ctx: *mut sg_ctx, dptr: *mut c_void) -> c_int;

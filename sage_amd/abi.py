@@ -59,6 +59,7 @@ _U64P = C.POINTER(C.c_uint64)
 # name -> (restype, argtypes): every symbol include/sage_hip.h declares
 PROTOTYPES = {
     "sg_ctx_create": (C.c_int, [C.c_int, C.c_uint64, C.POINTER(_CTX)]),
+    "sg_ctx_create_pooled": (C.c_int, [C.c_int, C.c_uint64, C.c_int, C.c_int, C.POINTER(_CTX)]),
     "sg_ctx_destroy": (C.c_int, [_CTX]),
     "sg_alloc": (C.c_int, [_CTX, C.c_uint64, C.POINTER(C.c_void_p)]),
     "sg_free": (C.c_int, [_CTX, C.c_void_p]),

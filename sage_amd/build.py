@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libsage_hip.so")
-SOURCES = ["runtime.cpp", "map_jit.cpp", "reduce.hip", "index.hip", "gemm.hip", "attention.hip", "rand.hip", "optim.hip"]
+SOURCES = ["runtime.cpp", "pool.cpp", "map_jit.cpp", "reduce.hip", "index.hip", "gemm.hip", "attention.hip", "rand.hip", "optim.hip"]
 # -packed-fp32-ops is switched off: hipcc would otherwise form v_pk_*_f32 from plain float code.
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -28,8 +28,26 @@ struct sg_map_entry {
     int result_dtype;
 };
 
+// The chunked allocator behind sg_ctx_create_pooled (Pool, memory.rs:199-475): free blocks of the two size classes,
+// each a range of one device allocation ("chunk"); blocks handed out are kept by address.
+struct sg_pool_block {
+    char *base;       // the chunk
+    uint64_t cap;     // bytes of the chunk
+    uint64_t size;    // bytes of this block
+    uint64_t offset;  // where it starts inside the chunk
+    uint64_t age;     // requests to its pool it has sat through (Counter, memory.rs:754-786)
+    bool whole() const { return size == cap; }  // !Block::is_split (memory.rs:749-751)
+};
+struct sg_pool {
+    bool sub_buffers = true;
+    std::vector<sg_pool_block> small, large;  // free blocks, in the order they were put back
+    std::unordered_map<void *, sg_pool_block> live;
+    uint64_t total = 0, used = 0, peak = 0;   // mem_total, mem_used, mem_peak (memory.rs:217-219)
+};
+
 // Context (session/context.rs:25-36): device + stream + kernel cache + allocator.
 struct sg_ctx {
+    sg_pool *pool = nullptr;  // set by sg_ctx_create_pooled with use_cache: sg_alloc / sg_free / sg_trim go through it
     int device = 0;
     hipStream_t stream = nullptr;
     int num_cus = 256;
@@ -115,6 +133,12 @@ static inline bool sg_is_dense(const sg_tensor *t) {
 }
 
 int sg_validate_tensor(sg_ctx *ctx, const sg_tensor *t, const char *name);
+
+// pool.cpp: the chunked allocator (sg_ctx::pool)
+int sg_pool_alloc(sg_ctx *ctx, uint64_t nbytes, void **dptr);
+int sg_pool_free(sg_ctx *ctx, void *dptr);
+int sg_pool_trim(sg_ctx *ctx);
+void sg_pool_destroy(sg_ctx *ctx);
 
 // gemm.hip: per-device set-up (the address of the static split-K scratch), run by sg_ctx_create.
 int sg_gemm_device_setup(sg_ctx *ctx);

@@ -86,8 +86,17 @@ int sg_ctx_create(int device_idx, uint64_t capacity_bytes, sg_ctx **out) {
     return SG_OK;
 }
 
+int sg_ctx_create_pooled(int device_idx, uint64_t capacity_bytes, int use_cache, int use_sub_buffer, sg_ctx **out) {
+    const int rc = sg_ctx_create(device_idx, capacity_bytes, out);
+    if (rc != SG_OK || !use_cache) return rc;
+    (*out)->pool = new sg_pool();
+    (*out)->pool->sub_buffers = use_sub_buffer != 0;
+    return SG_OK;
+}
+
 int sg_trim(sg_ctx *ctx) {
     if (!ctx) return SG_ERR_ARG;
+    if (ctx->pool) return sg_pool_trim(ctx);
     if (ctx->cache.empty()) return SG_OK;
     if (ctx->capturing) return sg_fail(ctx, SG_ERR_ARG, "sg_trim waits for the stream and cannot be captured into a graph");
     SG_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -106,6 +115,7 @@ int sg_ctx_destroy(sg_ctx *ctx) {
     for (auto &kv : ctx->jit) (void)hipModuleUnload(kv.second.module);
     for (auto &kv : ctx->cache) (void)hipFree(kv.second);
     for (auto &kv : ctx->live) (void)hipFree(kv.first);
+    sg_pool_destroy(ctx);
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return SG_OK;
@@ -121,6 +131,7 @@ static uint64_t round_block(uint64_t n) {
 int sg_alloc(sg_ctx *ctx, uint64_t nbytes, void **dptr) {
     if (!ctx || !dptr) return SG_ERR_ARG;
     *dptr = nullptr;
+    if (ctx->pool) return sg_pool_alloc(ctx, nbytes, dptr);
     // Pool::check_space (memory.rs:246-255)
     if (ctx->capacity && ctx->used + nbytes > ctx->capacity) {
         ctx->oom_needed = ctx->used + nbytes - ctx->capacity;
@@ -163,6 +174,7 @@ int sg_alloc(sg_ctx *ctx, uint64_t nbytes, void **dptr) {
 int sg_free(sg_ctx *ctx, void *dptr) {
     if (!ctx) return SG_ERR_ARG;
     if (!dptr) return SG_OK;
+    if (ctx->pool) return sg_pool_free(ctx, dptr);
     auto it = ctx->live.find(dptr);
     if (it == ctx->live.end()) return sg_fail(ctx, SG_ERR_ARG, "sg_free: %p was not allocated by this context", dptr);
     if (ctx->capturing) {
@@ -182,6 +194,13 @@ int sg_free(sg_ctx *ctx, void *dptr) {
 
 int sg_mem_stats(sg_ctx *ctx, uint64_t *used, uint64_t *reserved, uint64_t *peak, uint64_t *capacity) {
     if (!ctx) return SG_ERR_ARG;
+    if (ctx->pool) {
+        if (used) *used = ctx->pool->used;
+        if (reserved) *reserved = ctx->pool->total;
+        if (peak) *peak = ctx->pool->peak;
+        if (capacity) *capacity = ctx->capacity;
+        return SG_OK;
+    }
     if (used) *used = ctx->used;
     if (reserved) *reserved = ctx->reserved;
     if (peak) *peak = ctx->peak;

@@ -23,12 +23,15 @@ _PARAM_EPOCH = [0]
 
 class Context:
     """Context::with_device (context.rs:43-52).  capacity=None: bounded by the device only;
-    capacity=abi.REFERENCE_CAPACITY_BYTES reproduces the reference's 1000 MiB allocator cap."""
+    capacity=abi.REFERENCE_CAPACITY_BYTES reproduces the reference's 1000 MiB allocator cap.
+    use_cache / use_sub_buffer are the two switches of Allocator::new (memory.rs:64-69): the reference's Context
+    passes (False, True), every request then being a device allocation of its own; use_cache=True serves requests
+    from chunks (Pool's caching branch) and the capacity then bounds the bytes of the chunks held."""
 
-    def __init__(self, device=0, capacity=None):
+    def __init__(self, device=0, capacity=None, use_cache=False, use_sub_buffer=True):
         self._lib = abi.lib()
         h = C.c_void_p()
-        rc = self._lib.sg_ctx_create(int(device), int(capacity or 0), C.byref(h))
+        rc = self._lib.sg_ctx_create_pooled(int(device), int(capacity or 0), int(bool(use_cache)), int(bool(use_sub_buffer)), C.byref(h))
         if rc != abi.OK:
             raise abi.SageError(rc, f"sg_ctx_create(device={device}) failed: no usable HIP device")
         self.handle = h

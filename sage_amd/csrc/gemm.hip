@@ -309,7 +309,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     const float *R = p.res ? p.res + bt0 * p.r_sb0 + bt1 * p.r_sb1 : nullptr;
 
     // Direct epilogue (unguarded launches without activation or scaling): the accumulators START at bias[n] +
-    // residual[m][n] and leave, after the K loop, through buffer stores whose per-lane offset is fixed and whose
+    // residual[m][n] (neither costs a vector instruction once memory has answered) and leave, after the K loop, through buffer stores whose per-lane offset is fixed and whose
     // per-register offset is scalar -- no vector-ALU instruction and no LDS between the last MFMA and the last
     // store.  Vector-ALU work takes its cycles from the matrix pipe of the SIMD whichever wavefront issues it, so
     // only a write-out made of memory instructions alone can overlap the K loop of the next workgroup on the
@@ -321,10 +321,13 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     const uint32_t c_lane = ((uint32_t)(wm * WM + (lane >> 5) * 4) * (uint32_t)p.c_sm + (uint32_t)(wn * WN + (lane & 31))) * 4u;
     const uint32_t r_lane = ((uint32_t)(wm * WM + (lane >> 5) * 4) * (uint32_t)p.r_sm + (uint32_t)(wn * WN + (lane & 31))) * 4u;
     const __amdgpu_buffer_rsrc_t c_blk = __builtin_amdgcn_make_buffer_rsrc(C + (int64_t)m0 * p.c_sm + n0, 0, -1, 0x00020000);
+    uint32_t bias_lane = (lane >> 5) ? 0x80000000u : (uint32_t)(n0 + wn * WN + (lane & 31)) * 4u;
+    float bias_one = (lane >> 5) ? 0.0f : 1.0f;
+    asm volatile("" : "+v"(bias_lane), "+v"(bias_one));  // (formed here, among the early vector work, not where they are first used)
 
     // The requests are ordered so that nothing waits for memory twice: further down, the first two operand slabs,
-    // then the residual straight into the accumulator registers, then the bias (a handful of values), which is added
-    // once the first operands sit in LDS, right in front of the loop.
+    // then the residual straight into the accumulator registers, then the bias (a handful of values, added by the
+    // matrix pipe in front of the loop).
     floatx16 acc[TM][TN];
     float bias_j[TN];
 
@@ -567,8 +570,16 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
     }
+    {
+        // (lanes of the upper half, which stand for k = 1 of the MFMA below, ask beyond the descriptor's range and receive 0;
+        // so does every lane of a launch without a bias or with the staged epilogue, whose descriptor is empty: no branch
+        // here, whose outcome would have to travel to the MFMAs below through a vector register)
+        const __amdgpu_buffer_rsrc_t bias_d =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.bias ? p.bias : p.A), 0, direct && p.bias ? p.N * 4 : 0, 0x00020000);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) bias_j[j] = direct && p.bias ? p.bias[n0 + wn * WN + j * 32 + (lane & 31)] : 0.0f;
+        for (int j = 0; j < TN; ++j)
+            bias_j[j] = __builtin_bit_cast(float, (u32)__builtin_amdgcn_raw_buffer_load_b32(bias_d, bias_lane, (uint32_t)(j * 128), 0));
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int e = 0; e < NWR; ++e) SG_ITEM_STORE(e, ra0, rb0, 0);
@@ -577,13 +588,15 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     __syncthreads();
 #pragma unroll
     for (int e = 0; e < NRB; ++e) SG_ITEM_FETCH(e, 0, 0, a0, b0);
-    if (direct && p.bias) {
+    if (direct) {
+        // acc += ones x bias as one MFMA per block (A = 1 for k = 0 and 0 for k = 1, B = bias[n] for k = 0): the bias
+        // joins without a vector instruction.  Vector instructions of a workgroup that enters while an older one streams
+        // MFMAs get no issue slot; placed behind the first memory wait they would hold this workgroup's loop back until
+        // the older loop has ended (measured: 1.7 us of idle matrix pipe at the hand-over).
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[i][j][r] += bias_j[j];
+            for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bias_one, bias_j[j], acc[i][j], 0, 0, 0);
     }
     for (int kt = 0; kt < nk; kt += 2) {
         SG_SLAB_BODY(kt, ra1, rb1);

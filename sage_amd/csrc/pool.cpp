@@ -161,6 +161,11 @@ uint64_t release(sg_ctx *ctx, uint64_t size) {
 // Pool::alloc, caching branch (memory.rs:333-352)
 int sg_pool_alloc(sg_ctx *ctx, uint64_t nbytes, void **dptr) {
     sg_pool &p = *ctx->pool;
+    if (nbytes > (1ull << 48)) {  // (beyond any device; also keeps the roundings below from wrapping)
+        ctx->oom_needed = nbytes;
+        ctx->oom_total = p.total;
+        return sg_fail(ctx, SG_ERR_OOM, "tried to allocate %llu bytes", (unsigned long long)nbytes);
+    }
     const uint64_t size = (std::max<uint64_t>(nbytes, 1) + ALIGN - 1) / ALIGN * ALIGN;
     sg_pool_block b;
     if (!take_free_block(p, size, &b)) {

@@ -446,3 +446,47 @@ def test_relu_factor_is_read_from_the_output_outside_relu(monkeypatch):
     assert id(h2) in ev2.computed                       # the reference's graph stores the pre-activation
     assert ctx2._lib.log.count("sg_map") == with_rewrite + 1
     assert ctx2._lib.log.count("sg_gemm") + ctx2._lib.log.count("sg_matmul_strided") == ctx._lib.log.count("sg_gemm") + ctx._lib.log.count("sg_matmul_strided")
+
+
+def test_pool_model_keeps_an_allocators_invariants():
+    """The host-side model the GPU tests hold the chunked allocator against (tests/pool_model.py), on its own: blocks
+    handed out never overlap, every byte of every chunk is in exactly one block (handed out or free), free neighbours
+    never stay apart, the figures add up, and the capacity bounds the chunks held."""
+    import numpy as np
+    from tests import pool_model as PM
+    for seed, capacity, sub in [(0, 0, True), (1, 128 * PM.MIB, True), (2, 64 * PM.MIB, True), (3, 128 * PM.MIB, False)]:
+        rng = np.random.default_rng(seed)
+        m = PM.Pool(capacity, sub)
+        live = []
+        for step in range(1500):
+            if live and (rng.random() < 0.48 or len(live) > 60):
+                m.free(live.pop(int(rng.integers(len(live)))))
+            else:
+                r = rng.random()
+                n = int(rng.integers(1, 1 << 16)) if r < 0.4 else int(rng.integers(1 << 16, 3 << 20)) if r < 0.8 else int(rng.integers(3 << 20, 30 << 20))
+                try:
+                    chunk, off, size = m.alloc(n)
+                except PM.OutOfMemory:
+                    assert capacity, "an unbounded pool cannot run out"
+                    continue
+                assert size >= n and off % PM.ALIGN == 0
+                live.append((chunk, off))
+            blocks = [(b.chunk, b.offset, b.size, b.cap, "live") for b in m.live.values()]
+            blocks += [(b.chunk, b.offset, b.size, b.cap, "free") for b in m.small + m.large]
+            by_chunk = {}
+            for c, o, s, cap, kind in blocks:
+                by_chunk.setdefault(c, []).append((o, s, cap, kind))
+            total = 0
+            for c, parts in by_chunk.items():
+                parts.sort()
+                assert parts[0][0] == 0 and all(a[0] + a[1] == b[0] for a, b in zip(parts, parts[1:])), f"step {step}: chunk {c} has a hole or an overlap"
+                assert parts[-1][0] + parts[-1][1] == parts[0][2]
+                if sub:
+                    assert not any(a[3] == b[3] == "free" for a, b in zip(parts, parts[1:])), f"step {step}: free neighbours left apart"
+                total += parts[0][2]
+            assert total == m.total and m.used == sum(b.size for b in m.live.values()) and m.peak >= m.total
+            assert not capacity or m.total <= capacity
+        for k in live:
+            m.free(k)
+        m.trim()
+        assert m.used == 0 and m.total == 0 and not m.small and not m.large

@@ -661,6 +661,38 @@ def test_gemm_epilogues(ctx):
     close(y2.numpy(), 2.0 * (y1.numpy() - b), REL_GEMM, "shared")
 
 
+@pytest.mark.parametrize("with_res", [False, True])
+def test_gemm_direct_write_out_with_special_bias_values(ctx, with_res):
+    """Exactly tiled products without activation leave through the write-out that starts the accumulators at
+    bias + residual (the bias joins through the matrix pipe): infinities, NaN and huge values in the bias stay in
+    their own columns, everything else agrees with float64."""
+    say("direct write-out, special bias values, residual", with_res)
+    rng = np.random.default_rng(31)
+    m, k, n = 256, 96, 192
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (n,)).astype(np.float32)
+    bias[[0, 33, 95, 96, 191]] = [np.inf, -np.inf, np.nan, -0.0, 3e38]
+    res = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    lib = abi.lib()
+    ta, tb, tbias, tres = (S.Tensor.from_numpy(ctx, x) for x in (a, b, bias, res))
+    out = S.Tensor.uninit(ctx, [m, n])
+    ac, bc, oc, biasc, resc = ta.c(), tb.c(), out.c(), tbias.c(), tres.c()
+    epi = abi.sg_gemm_epilogue(1.0, abi.ACT_NONE, abi.ACT_NONE, C.pointer(biasc), C.pointer(resc) if with_res else None)
+    ctx.check(lib.sg_gemm(ctx.handle, 0, 0, C.byref(ac), C.byref(bc), C.byref(oc), C.byref(epi)))
+    name = C.create_string_buffer(128)
+    lib.sg_gemm_last_kernel_name(ctx.handle, name, 128)
+    assert b"false, false>" in name.value, f"expected an unguarded instantiation, got {name.value}"
+    got = out.numpy()
+    with np.errstate(all="ignore"):
+        want = a.astype(np.float64) @ b.astype(np.float64) + bias.astype(np.float64) + (res if with_res else 0.0)
+    assert np.all(got[:, 0] == np.inf) and np.all(got[:, 33] == -np.inf) and np.all(np.isnan(got[:, 95]))
+    assert np.all(np.isfinite(got[:, 191])) and np.allclose(got[:, 191], 3e38, rtol=1e-6)
+    ok = np.ones(n, bool)
+    ok[[0, 33, 95, 191]] = False
+    close(got[:, ok], want[:, ok], REL_GEMM, "finite columns")
+
+
 # ----------------------------------------------------------------------------- conv
 IM2COL_CASES = [
     ((2, 28, 28, 1), 7, 2, 3, 1), ((2, 14, 14, 64), 3, 2, 1, 1), ((3, 7, 7, 64), 3, 1, 1, 1), ((2, 7, 7, 64), 1, 2, 0, 1),

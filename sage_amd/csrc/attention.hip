@@ -62,9 +62,9 @@ struct AttnP {
 // scalar fallbacks.  A launch starts with a cold instruction cache, and what a workgroup executes before its
 // first MFMA is fetched line by line: at b32 x 12 heads x s128 the prologue (pointer arithmetic with two
 // integer divisions, eight guarded and doubly coded Q loads, the first K/V requests) took 6 of the kernel's
-// 22 us.  Hence: divisions by multiply-high, row indices clamped instead of guarded (a query past the end
-// computes on the last row and is not written; a key past the end reads the last row and is masked with
-// -inf), one code path per load.
+// 22 us.  Hence: divisions by multiply-high, no guards (a query past the end computes on the last row and is
+// not written; a key past the end reads as zeros through the buffer descriptor's range check and is masked
+// with -inf), one code path per load, K and V requested through buffer loads with fixed per-lane offsets.
 __device__ __forceinline__ uint32_t fdiv(uint32_t n, sg_fastdiv d) { return (__umulhi(n, d.magic) + n) >> d.shift; }
 
 template <int D, bool SPLIT, bool VEC>
@@ -114,17 +114,41 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((S
     // global -> registers for one K/V block; piece f of the block: row f / ROWV, floats 4*(f % ROWV)..
     f32x4 kreg[NLD], vreg[NLD];
     float mreg = 0.0f;
+    // VEC: the K and V requests are buffer loads: a descriptor per (batch, head) that ends behind the last key's row,
+    // a per-lane byte offset fixed for the kernel (the piece's row and column inside a block) and a scalar offset per
+    // block.  No address arithmetic on the vector unit in the key loop (it was a quarter of the loop's vector
+    // instructions, and every one of them is paid in matrix-pipe cycles); a key past the end lies beyond the
+    // descriptor's range and reads as zeros, its mask is -inf.
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    uint32_t koff[NLD], voff[NLD];
+    __amdgpu_buffer_rsrc_t kdesc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(K), 0, 0, 0x00020000), vdesc = kdesc;
+    if (VEC) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int f = tid + i * 64 * NW;
+            const int row = f / ROWV, c = (f % ROWV) * 4;
+            koff[i] = ((uint32_t)row * (uint32_t)p.k_sl + (uint32_t)c) * 4u;
+            voff[i] = ((uint32_t)row * (uint32_t)p.v_sl + (uint32_t)c) * 4u;
+        }
+        kdesc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(K), 0, (int)(((uint32_t)(p.Lk - 1) * (uint32_t)p.k_sl + (uint32_t)D) * 4u), 0x00020000);
+        vdesc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(V), 0, (int)(((uint32_t)(p.Lk - 1) * (uint32_t)p.v_sl + (uint32_t)D) * 4u), 0x00020000);
+    }
     auto request = [&](int kb0) {
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
+            if (VEC) {
+                kreg[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_amdgcn_raw_buffer_load_b128(kdesc, koff[i], (uint32_t)kb0 * (uint32_t)p.k_sl * 4u, 0));
+                vreg[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_amdgcn_raw_buffer_load_b128(vdesc, voff[i], (uint32_t)kb0 * (uint32_t)p.v_sl * 4u, 0));
+                continue;
+            }
             const int f = tid + i * 64 * NW;
             const int row = f / ROWV, c = (f % ROWV) * 4;
             const int key = min(kb0 + row, p.Lk - 1);  // a key past the end repeats the last one (finite values); its mask is -inf
             const float *kp = K + (int64_t)key * p.k_sl + c, *vp = V + (int64_t)key * p.v_sl + c;
             f32x4 a, b;
-            if (VEC || p.vec_k) a = *reinterpret_cast<const f32x4 *>(kp);
+            if (p.vec_k) a = *reinterpret_cast<const f32x4 *>(kp);
             else { a.x = kp[0]; a.y = kp[1]; a.z = kp[2]; a.w = kp[3]; }
-            if (VEC || p.vec_v) b = *reinterpret_cast<const f32x4 *>(vp);
+            if (p.vec_v) b = *reinterpret_cast<const f32x4 *>(vp);
             else { b.x = vp[0]; b.y = vp[1]; b.z = vp[2]; b.w = vp[3]; }
             kreg[i] = a;
             vreg[i] = b;
@@ -388,7 +412,9 @@ extern "C" int sg_attention(sg_ctx *ctx, const sg_tensor *q, const sg_tensor *k,
     p.xcd_remap = grid.x > 1 && (grid.x * grid.y) % 8 == 0;
     p.d_gx = sg_make_fastdiv(grid.x);
     p.d_nb1 = sg_make_fastdiv((uint32_t)nb1);
-    const bool vec = p.vec_q && p.vec_k && p.vec_v && p.vec_o;
+    // the all-aligned instantiation addresses K and V through 32-bit byte offsets from the (batch, head) pair's first row
+    const bool fits32 = (Lk + 64) * p.k_sl < (1ll << 29) && (Lk + 64) * p.v_sl < (1ll << 29) && p.k_sl >= 0 && p.v_sl >= 0;
+    const bool vec = p.vec_q && p.vec_k && p.vec_v && p.vec_o && fits32;
 #define SG_ATTN_LAUNCH(D_, SPLIT_)                                                                                             \
     do {                                                                                                                       \
         if (vec) hipLaunchKernelGGL((attention_kernel<D_, SPLIT_, true>), grid, dim3(64 * NW), 0, ctx->stream, p);            \

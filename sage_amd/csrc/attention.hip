@@ -246,7 +246,8 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((S
         const float mshift = -m_new * LOG2E;
         // the shift rarely moves after the first blocks: when it stayed put for every query of the wavefront the
         // correction factor is exactly 1 and rescaling the accumulators (vector work the matrix pipe waits for) is skipped
-        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+        // (nothing to rescale in front of the first block: the accumulators and the sum are still zero)
+        if (kb0 > 0 && __builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
             const float corr = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
             l_run *= corr;
 #pragma unroll
@@ -305,8 +306,13 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((S
         const float *src = &lds_k[(wave * 64 + lane) * SLOT];
         const float m_b = src[16 * ND], l_b = src[16 * ND + 1];
         const float m = fmaxf(m_run, m_b);
-        const float ca = __builtin_amdgcn_exp2f((m_run - m) * LOG2E), cb = __builtin_amdgcn_exp2f((m_b - m) * LOG2E);
+        float ca = __builtin_amdgcn_exp2f((m_run - m) * LOG2E), cb = __builtin_amdgcn_exp2f((m_b - m) * LOG2E);
         l_run = l_run * ca + l_b * cb;
+        // the 1/l of the normalisation below rides on the two merge factors: one multiplication per value less
+        const float lm = l_run + __shfl_xor(l_run, 32, 64);
+        const float invm = 1.0f / lm;
+        ca *= invm;
+        cb *= invm;
 #pragma unroll
         for (int j = 0; j < ND; ++j)
 #pragma unroll
@@ -315,7 +321,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((S
     // ---- normalise and write: register r = 4g + s of block j is head index ND*(8g + 4h + s) + j, so the
     // 4*ND values of one g are consecutive head indices starting at ND*(8g + 4h)
     const float l = l_run + __shfl_xor(l_run, 32, 64);
-    const float inv = 1.0f / l;
+    const float inv = SPLIT ? 1.0f : 1.0f / l;
     const int q = q0 + ql;
     if (q < p.Lq) {
         float *row = p.o + bt0 * p.o_sb0 + bt1 * p.o_sb1 + (int64_t)q * p.o_sl;

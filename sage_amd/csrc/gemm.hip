@@ -951,8 +951,7 @@ int launch_cfg(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noal
     }
     // one workgroup per tile while they all fit at once (three per compute unit), else that many workgroups
     // walking the tiles; a batched product keeps one workgroup per tile and batch entry
-    static const int res_per_cu = getenv("SAGE_GEMM_RESIDENT") ? atoi(getenv("SAGE_GEMM_RESIDENT")) : 3;  // EXPERIMENT
-    const int64_t ntiles = (int64_t)p.tiles_m * p.tiles_n, resident = res_per_cu * (int64_t)ctx->num_cus;
+    const int64_t ntiles = (int64_t)p.tiles_m * p.tiles_n, resident = 3 * (int64_t)ctx->num_cus;
     dim3 grid((unsigned)(batch == 1 && ntiles > resident ? resident : ntiles), (unsigned)batch);
     set_direct(ctx, p, BM);
     if (needs_guard(p, BM, BN, a_kc, b_nc)) launch_layouts<BM, BN, WAVES_M, true>(ctx, p, grid, a_kc, b_nc);

@@ -29,9 +29,10 @@
 //     run of MFMAs).  Hence no vector address arithmetic in the K loop -- global requests are buffer
 //     loads with fixed per-lane offsets, LDS reads take fixed per-lane origins plus immediates (nine
 //     address additions per two slabs, which the compiler had placed there for paired LDS reads, cost
-//     6 % of a 128x96 loop: 1640 cycles per slab against the 1536 of its 24 MFMAs, now 1539) -- a short
-//     branch-free erf in the GELU epilogue, and workgroups that walk tiles (the loops of the workgroups
-//     on a compute unit run one after the other anyway).
+//     6 % of a 128x96 loop: 1640 cycles per slab against the 1536 of its 24 MFMAs, now 1539) -- a GELU
+//     epilogue that reads the normal distribution function from a table in LDS (nine vector
+//     instructions per value), and workgroups that walk tiles (the loops of the workgroups on a
+//     compute unit run one after the other anyway).
 //   * Workgroup ids are remapped so that the ids one XCD receives (id mod 8) cover a compact block
 //     of tiles, which keeps the A/B panels a tile group shares inside that XCD's L2.
 //   * The epilogue applies alpha, bias[n], activation and a residual on the way out: accumulator
@@ -46,6 +47,7 @@
 #include "common.h"
 
 #include <atomic>
+#include <cmath>
 #include <type_traits>
 
 namespace {
@@ -65,6 +67,19 @@ constexpr int64_t SCRATCH_FLOATS = (int64_t)SG_GEMM_NOALLOC_SCRATCH_BYTES / 4;
 static __device__ __align__(256) float scratch[SCRATCH_FLOATS];
 constexpr int MAX_DEVICES = 64;
 std::atomic<float *> g_scratch_ptr[MAX_DEVICES];  // device address of `scratch` on each GPU (zero-initialised), set by sg_gemm_device_setup
+
+// The standard normal distribution function on [-6, 6) as 384 cubic pieces (Hermite: exact values and slopes at the
+// nodes, worked out in double precision when a device is set up), for the GELU epilogue of the product kernels:
+// x * Phi(x) = 0.5 x (1 + erf(x / sqrt 2)).  Piece i covers [-6 + i/32, -6 + (i+1)/32) and holds the coefficients of
+// c0 + t (c1 + t (c2 + t c3)), t in [0, 1): the interpolation error is below 2e-9, so what is left is fp32 rounding
+// (|error of x Phi(x)| < 5e-7 over [-8, 8], the size of half an ulp of x there).  Nine vector instructions and one
+// 16-byte LDS read per value against seventeen for the rational-exponential erf below, and in an epilogue every
+// vector instruction is a cycle taken from the matrix pipe.  Below -6 the table's first value is 0 (the product is
+// -0, the limit), above 6 its last is 1.
+constexpr int GELU_PIECES = 384;
+constexpr int GELU_TAB_BYTES = GELU_PIECES * 16;
+static __device__ __align__(256) float gelu_tab[GELU_PIECES * 4];
+std::atomic<float *> g_gelu_tab_ptr[MAX_DEVICES];  // device address of `gelu_tab` on each GPU, set by sg_gemm_device_setup
 
 // Convolution as a GEMM whose A operand is never materialised: row m of A is output pixel
 // (n, oh, ow), column k is filter tap and channel (ky, kx, c), and A[m][k] is read from the image
@@ -95,6 +110,7 @@ struct GemmP {
     int vec_c, vec_r, vec_bias;  // 16-byte accesses are legal for C rows / residual rows / the bias
     int direct;       // epilogue without vector-ALU work is legal (set by the host, see the kernel): no activation, alpha = 1,
                       // every C / residual offset inside a tile below 2^31 bytes, unguarded instantiation
+    const float *gelu;  // the table above when an activation of this launch is GELU (the kernel then has GELU_TAB_BYTES of dynamic LDS), else null
     int k_chunk;      // split-K: workgroup z multiplies k in [z*k_chunk, min(K, (z+1)*k_chunk)); 0 = all of K
     int64_t c_sz;     // split-K: element stride between the partial results of consecutive z
     ConvG conv;       // used by the CONV instantiations only (A is then the image)
@@ -105,8 +121,8 @@ struct GemmP {
 // with the hardware reciprocal and 2^x.  Absolute error below 6e-7 in fp32 (1.5e-7 from the formula, the
 // rest from forming 1 - small in fp32): three orders of magnitude inside the tolerance of a GEMM-bearing
 // result.  A dozen instructions, no branch, against about forty with two divergent paths for the
-// library routine; in an epilogue every vector instruction is a cycle taken from the matrix pipe.
-// The map kernels keep the exact routine.
+// library routine.  Used where no table is at hand: the split-K second pass and the one-row-per-wavefront kernel
+// (the tiled kernels read the table above; the map kernels keep the exact routine).
 __device__ __forceinline__ float erf_short(float x) {
     const float ax = __builtin_fabsf(x);
     const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f, ax, 1.0f));
@@ -124,8 +140,19 @@ __device__ __forceinline__ float apply_act(float v, int act) {
     if (act == SG_ACT_GELU_ERF) return (v * 0.5f) * (erf_short(v * 0.70710678118654752440f) + 1.0f);
     return v;
 }
+// GELU through the table (in LDS, 16 bytes per piece)
+__device__ __forceinline__ float gelu_lookup(float x, const float *tab) {
+    const float u = __builtin_amdgcn_fmed3f(__builtin_fmaf(x, 32.0f, 192.0f), 0.0f, 383.99997f);
+    const float t = __builtin_amdgcn_fractf(u);
+    const f32x4 c = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const char *>(tab) + ((uint32_t)(int)u << 4));
+    return x * __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(c.w, t, c.z), t, c.y), t, c.x);
+}
 // the same for the four values of a lane, with one uniform branch on the kind instead of four
-__device__ __forceinline__ void apply_act4(f32x4 &v, int act) {
+__device__ __forceinline__ void apply_act4(f32x4 &v, int act, const float *gelu_lds) {
+    if (act == SG_ACT_GELU_ERF && gelu_lds) {
+        v.x = gelu_lookup(v.x, gelu_lds); v.y = gelu_lookup(v.y, gelu_lds); v.z = gelu_lookup(v.z, gelu_lds); v.w = gelu_lookup(v.w, gelu_lds);
+        return;
+    }
     if (act == SG_ACT_RELU) {
         v.x = apply_act(v.x, SG_ACT_RELU); v.y = apply_act(v.y, SG_ACT_RELU); v.z = apply_act(v.z, SG_ACT_RELU); v.w = apply_act(v.w, SG_ACT_RELU);
     } else if (act == SG_ACT_GELU_ERF) {
@@ -264,6 +291,23 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     constexpr int LDS_FLOATS = LDS_OPERANDS > 4 * STAGE ? LDS_OPERANDS : 4 * STAGE;
     __shared__ __attribute__((aligned(16))) float lds_raw[LDS_FLOATS];
     float(*lds_a)[TA::SIZE] = reinterpret_cast<float(*)[TA::SIZE]>(lds_raw);
+    // GELU launches carry the table in dynamic LDS behind the buffers above: every wavefront brings its share (64 pieces
+    // per request) with loads that write LDS directly, no register in between; they are the first requests of the
+    // kernel, so the wait for the first operand slab and the barrier behind it also make the table visible.
+    extern __shared__ __attribute__((aligned(16))) float gelu_dyn[];
+    const float *gelu_lds = nullptr;
+    if (p.gelu) {
+        gelu_lds = gelu_dyn;
+        const __amdgpu_buffer_rsrc_t tab_d = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.gelu), 0, GELU_TAB_BYTES, 0x00020000);
+        const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        typedef __attribute__((address_space(3))) void *lds_ptr;
+#pragma unroll
+        for (int r = 0; r < (GELU_PIECES + NTHREADS - 1) / NTHREADS; ++r) {
+            const int first = r * NTHREADS + w * 64;  // this wavefront's first piece of round r
+            if (first < GELU_PIECES)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(tab_d, (lds_ptr)(gelu_dyn + first * 4), 16, (uint32_t)((first + (threadIdx.x & 63)) * 16), 0, 0, 0);
+        }
+    }
     float(*lds_b)[TB::SIZE] = reinterpret_cast<float(*)[TB::SIZE]>(lds_raw + 2 * TA::SIZE);
 
     // ---- which tile: spread consecutive ids over XCDs, then walk tiles in groups of 8 tile-rows
@@ -700,9 +744,9 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
                 if (GUARD && (m >= p.M || n >= p.N)) continue;
                 if (p.alpha != 1.0f) v *= p.alpha;
                 if (p.bias) v += bias_c;
-                if (ACT) apply_act4(v, p.act);
+                if (ACT) apply_act4(v, p.act, gelu_lds);
                 if (R) v += res;
-                if (ACT) apply_act4(v, p.act_post);
+                if (ACT) apply_act4(v, p.act_post, gelu_lds);
                 float *cp = C + (int64_t)m * p.c_sm + n;
                 if (!GUARD || (p.vec_c && n_in)) *reinterpret_cast<f32x4 *>(cp) = v;
                 else {
@@ -832,19 +876,23 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const GemmP p) {
 }
 
 template <int BM, int BN, int WAVES_M, bool GUARD>
-void launch_layouts(sg_ctx *ctx, const GemmP &p, dim3 grid, bool a_kc, bool b_nc) {
+void launch_layouts(sg_ctx *ctx, const GemmP &p_in, dim3 grid, bool a_kc, bool b_nc) {
+    GemmP p = p_in;
+    const bool gelu = p.act == SG_ACT_GELU_ERF || p.act_post == SG_ACT_GELU_ERF;
+    p.gelu = gelu && ctx->device >= 0 && ctx->device < MAX_DEVICES ? g_gelu_tab_ptr[ctx->device].load(std::memory_order_acquire) : nullptr;
     dim3 block(NTHREADS);
+    const unsigned dyn = p.gelu ? GELU_TAB_BYTES : 0;
     const bool conv = p.conv.ohw != 0;
     const int inst[7] = {BM, BN, WAVES_M, conv || a_kc, conv || b_nc, GUARD, conv};
     for (int i = 0; i < 7; ++i) ctx->last_gemm[i] = inst[i];
     if (conv) {  // image-addressed A (sg_conv2d): one instantiation per tile shape
-        hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD, true>), grid, block, 0, ctx->stream, p);
+        hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD, true>), grid, block, dyn, ctx->stream, p);
         return;
     }
-    if (a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD>), grid, block, 0, ctx->stream, p);
-    else if (a_kc && !b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, false, GUARD>), grid, block, 0, ctx->stream, p);
-    else if (!a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, true, GUARD>), grid, block, 0, ctx->stream, p);
-    else hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, false, GUARD>), grid, block, 0, ctx->stream, p);
+    if (a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD>), grid, block, dyn, ctx->stream, p);
+    else if (a_kc && !b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, false, GUARD>), grid, block, dyn, ctx->stream, p);
+    else if (!a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, true, GUARD>), grid, block, dyn, ctx->stream, p);
+    else hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, false, GUARD>), grid, block, dyn, ctx->stream, p);
 }
 
 // The epilogue made of buffer stores alone (see the kernel): no activation, no scaling, and every offset inside a
@@ -1232,7 +1280,25 @@ extern "C" int sg_conv2d(sg_ctx *ctx, const sg_tensor *x, const sg_tensor *filte
 // on that GPU once (each GPU holds its own copy of the array at its own address).
 int sg_gemm_device_setup(sg_ctx *ctx) {
     if (ctx->device < 0 || ctx->device >= MAX_DEVICES) return SG_OK;  // sg_gemm_noalloc reports it when used
-    if (g_scratch_ptr[ctx->device].load(std::memory_order_acquire)) return SG_OK;
+    if (g_scratch_ptr[ctx->device].load(std::memory_order_acquire) && g_gelu_tab_ptr[ctx->device].load(std::memory_order_acquire)) return SG_OK;
+    if (!g_gelu_tab_ptr[ctx->device].load(std::memory_order_acquire)) {
+        static float host_tab[GELU_PIECES * 4];  // (the same values whichever thread writes them)
+        const double h = 1.0 / 32.0;
+        auto Phi = [](double x) { return 0.5 * erfc(-x * 0.70710678118654752440); };
+        auto phi = [](double x) { return exp(-0.5 * x * x) * 0.39894228040143267794; };
+        for (int i = 0; i < GELU_PIECES; ++i) {
+            const double x0 = -6.0 + i * h, x1 = x0 + h;
+            const double v0 = i == 0 ? 0.0 : Phi(x0), v1 = Phi(x1), s0 = phi(x0) * h, s1 = phi(x1) * h, d = v1 - v0;
+            host_tab[4 * i + 0] = (float)v0;
+            host_tab[4 * i + 1] = (float)s0;
+            host_tab[4 * i + 2] = (float)(3.0 * d - 2.0 * s0 - s1);
+            host_tab[4 * i + 3] = (float)(s0 + s1 - 2.0 * d);
+        }
+        SG_HIP(ctx, hipMemcpyToSymbol(HIP_SYMBOL(gelu_tab), host_tab, sizeof host_tab));
+        float *tab = nullptr;
+        SG_HIP(ctx, hipGetSymbolAddress((void **)&tab, HIP_SYMBOL(gelu_tab)));
+        g_gelu_tab_ptr[ctx->device].store(tab, std::memory_order_release);
+    }
     float *ptr = nullptr;
     SG_HIP(ctx, hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
     // contexts created at the same time on several threads all resolve the same address: whichever store lands is right

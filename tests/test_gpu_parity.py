@@ -693,6 +693,41 @@ def test_gemm_direct_write_out_with_special_bias_values(ctx, with_res):
     close(got[:, ok], want[:, ok], REL_GEMM, "finite columns")
 
 
+@pytest.mark.parametrize("m,n", [(128, 96), (256, 128), (100, 70)])
+def test_gemm_gelu_epilogue_over_the_whole_range(ctx, m, n):
+    """The product kernels' GELU (a table of cubic pieces of the normal distribution function in LDS) against float64
+    0.5 x (1 + erf(x / sqrt 2)): over [-9, 9], at the table's nodes and ends, far outside it, on zeros, infinities and NaN.
+    The pre-activations are exact: y = gelu(X . I), every product with one non-zero term."""
+    import math
+    say("gelu epilogue", m, n)
+    rng = np.random.default_rng(41)
+    vals = np.concatenate([np.linspace(-9, 9, 4001), -6 + np.arange(0, 385) / 32, [-6.0001, 5.99999, 6.0, 6.0001, -100, 100, -1e30, 1e30, 0.0, -0.0, 1e-30, -1e-30],
+                           rng.standard_normal(4000) * 2]).astype(np.float32)
+    x = np.resize(vals, m * n).reshape(m, n)
+    lib = abi.lib()
+    tx, teye, to = S.Tensor.from_numpy(ctx, x), S.Tensor.from_numpy(ctx, np.eye(n, dtype=np.float32)), S.Tensor.uninit(ctx, [m, n])
+    xc, eyec, oc = tx.c(), teye.c(), to.c()
+    epi = abi.sg_gemm_epilogue(1.0, abi.ACT_GELU_ERF, abi.ACT_NONE, None, None)
+    ctx.check(lib.sg_gemm(ctx.handle, 0, 0, C.byref(xc), C.byref(eyec), C.byref(oc), C.byref(epi)))
+    got = to.numpy()
+    xf = x.astype(np.float64)
+    want = 0.5 * xf * (1.0 + np.vectorize(math.erf)(xf / math.sqrt(2.0)))
+    err = np.abs(got - want)
+    bound = 6e-7 * np.maximum(1.0, np.abs(xf))
+    worst = np.unravel_index(np.argmax(err - bound), err.shape)
+    assert np.all(err <= bound), f"gelu({x[worst]}) = {got[worst]}, float64 {want[worst]}"
+    # infinities and NaN arrive through the bias (as operands of the product they would spread over their rows)
+    special = np.array([np.inf, -np.inf, np.nan, -0.0] + [0.0] * (n - 4), np.float32)
+    tz, tbias = S.Tensor.from_numpy(ctx, np.zeros((m, n), np.float32)), S.Tensor.from_numpy(ctx, special)
+    zc, biasc = tz.c(), tbias.c()
+    epi = abi.sg_gemm_epilogue(1.0, abi.ACT_GELU_ERF, abi.ACT_NONE, C.pointer(biasc), None)
+    ctx.check(lib.sg_gemm(ctx.handle, 0, 0, C.byref(zc), C.byref(eyec), C.byref(oc), C.byref(epi)))
+    got = to.numpy()
+    # (-inf times the 0 it approaches is NaN in the reference's 0.5 x (1 + erf) as well)
+    assert np.all(got[:, 0] == np.inf) and np.all(np.isnan(got[:, 1])) and np.all(np.isnan(got[:, 2])), got[0, :4]
+    assert np.all(got[:, 3:] == 0.0)
+
+
 # ----------------------------------------------------------------------------- conv
 IM2COL_CASES = [
     ((2, 28, 28, 1), 7, 2, 3, 1), ((2, 14, 14, 64), 3, 2, 1, 1), ((3, 7, 7, 64), 3, 1, 1, 1), ((2, 7, 7, 64), 1, 2, 0, 1),

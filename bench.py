@@ -335,7 +335,7 @@ def kernel_workloads(ctx, name, rng, elements=None):
         M = N = K = 4096
         A, Bm, bias = (dev(rng.uniform(-1, 1, s).astype(np.float32)) for s in ((M, K), (K, N), (N,)))
         progs = programs(lambda i: A.matmul(Bm) + bias, 2)
-        return progs, 4.0 * (M * K + K * N + M * N + N), 2.0 * M * N * K + M * N, "gemm_mfma_kernel<128, 128, 2, true, true, false, false>", ("gemm", M, N, K)
+        return progs, 4.0 * (M * K + K * N + M * N + N), 2.0 * M * N * K + M * N, "gemm_mfma_kernel<128, 128, 2, true, true, false, false, true>", ("gemm", M, N, K)
     raise SystemExit(f"unknown workload {name}")
 
 

@@ -258,8 +258,8 @@ int sg_matmul_strided(sg_ctx *ctx, const sg_tensor *a, const sg_tensor *b, const
 
 /* Name of the kernel instantiation the most recent product on this context launched (sg_gemm,
  * sg_gemm_batched, sg_matmul_strided, sg_conv2d; for a split-K product: its first pass), as it appears
- * in a rocprofv3 kernel trace: tile sizes, operand layouts, guarded loads and image addressing are
- * template arguments.  The reference has one fixed 8x8 kernel per transpose mode (gemm.rs:208-221);
+ * in a rocprofv3 kernel trace: tile sizes, operand layouts, guarded loads, image addressing and the kind of
+ * write-out are template arguments.  The reference has one fixed 8x8 kernel per transpose mode (gemm.rs:208-221);
  * here the instantiation is chosen per shape.  SG_ERR_ARG before the first product. */
 int sg_gemm_last_kernel_name(sg_ctx *ctx, char *buf, uint64_t cap);
 

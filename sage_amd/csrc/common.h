@@ -73,7 +73,7 @@ struct sg_ctx {
     // SAGE_ATTENTION_SPLIT (0/1, -1 = the heuristic), SAGE_GEMM_DIRECT (0 = staged epilogue only).
     int force_gemm_split = 0, force_gemm_tile = -1, force_attention_split = -1;
     int gemm_direct = 1;  // SAGE_GEMM_DIRECT=0: products always leave through the staged epilogue
-    int last_gemm[7] = {0, 0, 0, 0, 0, 0, 0};  // template arguments of the most recent product kernel (BM 0: none yet)
+    int last_gemm[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // template arguments of the most recent product kernel (BM 0: none yet)
     std::vector<void *> capture_allocs, capture_held;
     // errors
     std::string last_error;

@@ -276,9 +276,10 @@ template <int ROWS, bool K_CONTIG> struct Tile {
 
 __device__ __forceinline__ uint32_t fdiv(uint32_t n, sg_fastdiv d) { return (__umulhi(n, d.magic) + n) >> d.shift; }
 
-template <int BM, int BN, int WAVES_M, bool A_KC, bool B_NC, bool GUARD, bool CONV = false>
+template <int BM, int BN, int WAVES_M, bool A_KC, bool B_NC, bool GUARD, bool CONV = false, bool DIRECT = false>
 __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3, 8))) gemm_mfma_kernel(const GemmP p) {
     static_assert(!CONV || A_KC, "the image-addressed A operand is k-contiguous");
+    static_assert(!DIRECT || !GUARD, "the direct write-out belongs to the unguarded instantiations");
     constexpr int WAVES_N = 4 / WAVES_M;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -359,7 +360,7 @@ __global__ void __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(3
     // only a write-out made of memory instructions alone can overlap the K loop of the next workgroup on the
     // compute unit (or of this workgroup's next tile).  Element r of a 32x32 accumulator block is row
     // (r/4)*8 + (lane/32)*4 + r%4, column lane%32: a store instruction writes two full 128-byte row segments.
-    const bool direct = !GUARD && p.direct;
+    constexpr bool direct = DIRECT;  // (an instantiation of its own: a kernel holds one of the two write-outs, not both)
     typedef unsigned int u32;
     // (descriptors are per tile, hence uniform; the wavefront's block inside the tile is part of the per-lane offset)
     const uint32_t c_lane = ((uint32_t)(wm * WM + (lane >> 5) * 4) * (uint32_t)p.c_sm + (uint32_t)(wn * WN + (lane & 31))) * 4u;
@@ -875,6 +876,18 @@ __global__ void __launch_bounds__(256) gemm_skinny_kernel(const GemmP p) {
     }
 }
 
+template <int BM, int BN, int WAVES_M, bool GUARD, bool DIRECT>
+void launch_variants(sg_ctx *ctx, const GemmP &p, dim3 grid, dim3 block, unsigned dyn, bool conv, bool a_kc, bool b_nc) {
+    if (conv) {  // image-addressed A (sg_conv2d): one instantiation per tile shape
+        hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD, true, DIRECT>), grid, block, dyn, ctx->stream, p);
+        return;
+    }
+    if (a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD, false, DIRECT>), grid, block, dyn, ctx->stream, p);
+    else if (a_kc && !b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, false, GUARD, false, DIRECT>), grid, block, dyn, ctx->stream, p);
+    else if (!a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, true, GUARD, false, DIRECT>), grid, block, dyn, ctx->stream, p);
+    else hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, false, GUARD, false, DIRECT>), grid, block, dyn, ctx->stream, p);
+}
+
 template <int BM, int BN, int WAVES_M, bool GUARD>
 void launch_layouts(sg_ctx *ctx, const GemmP &p_in, dim3 grid, bool a_kc, bool b_nc) {
     GemmP p = p_in;
@@ -883,16 +896,16 @@ void launch_layouts(sg_ctx *ctx, const GemmP &p_in, dim3 grid, bool a_kc, bool b
     dim3 block(NTHREADS);
     const unsigned dyn = p.gelu ? GELU_TAB_BYTES : 0;
     const bool conv = p.conv.ohw != 0;
-    const int inst[7] = {BM, BN, WAVES_M, conv || a_kc, conv || b_nc, GUARD, conv};
-    for (int i = 0; i < 7; ++i) ctx->last_gemm[i] = inst[i];
-    if (conv) {  // image-addressed A (sg_conv2d): one instantiation per tile shape
-        hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD, true>), grid, block, dyn, ctx->stream, p);
-        return;
+    const bool direct = !GUARD && p.direct;
+    const int inst[8] = {BM, BN, WAVES_M, conv || a_kc, conv || b_nc, GUARD, conv, direct};
+    for (int i = 0; i < 8; ++i) ctx->last_gemm[i] = inst[i];
+    if constexpr (!GUARD) {
+        if (direct) {
+            launch_variants<BM, BN, WAVES_M, false, true>(ctx, p, grid, block, dyn, conv, a_kc, b_nc);
+            return;
+        }
     }
-    if (a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, true, GUARD>), grid, block, dyn, ctx->stream, p);
-    else if (a_kc && !b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, true, false, GUARD>), grid, block, dyn, ctx->stream, p);
-    else if (!a_kc && b_nc) hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, true, GUARD>), grid, block, dyn, ctx->stream, p);
-    else hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WAVES_M, false, false, GUARD>), grid, block, dyn, ctx->stream, p);
+    launch_variants<BM, BN, WAVES_M, GUARD, false>(ctx, p, grid, block, dyn, conv, a_kc, b_nc);
 }
 
 // The epilogue made of buffer stores alone (see the kernel): no activation, no scaling, and every offset inside a
@@ -1050,8 +1063,8 @@ int launch_gemm(sg_ctx *ctx, GemmP &p, int batch, bool a_kc, bool b_nc, bool noa
     // in MFMA tiles: 1024 x 512 x 16 took 18 us, 32768 x 768 x 2 43 us)
     if (batch == 1 && p.conv.ohw == 0 && p.N <= 16 && p.M <= 512 && ctx->force_gemm_tile < 0 && ctx->force_gemm_split == 0) {
         dim3 grid((unsigned)((p.M + 3) / 4));
-        const int inst[7] = {-1, p.N <= 4 ? 4 : 16, 0, 0, 0, 0, 0};  // sg_gemm_last_kernel_name: gemm_skinny_kernel<NMAX>
-        for (int i = 0; i < 7; ++i) ctx->last_gemm[i] = inst[i];
+        const int inst[8] = {-1, p.N <= 4 ? 4 : 16, 0, 0, 0, 0, 0, 0};  // sg_gemm_last_kernel_name: gemm_skinny_kernel<NMAX>
+        for (int i = 0; i < 8; ++i) ctx->last_gemm[i] = inst[i];
         if (p.N <= 4) hipLaunchKernelGGL((gemm_skinny_kernel<4>), grid, dim3(256), 0, ctx->stream, p);
         else hipLaunchKernelGGL((gemm_skinny_kernel<16>), grid, dim3(256), 0, ctx->stream, p);
         SG_CHECK_LAUNCH(ctx, "gemm (skinny)");
@@ -1160,8 +1173,8 @@ extern "C" int sg_gemm_last_kernel_name(sg_ctx *ctx, char *buf, uint64_t cap) {
         snprintf(buf, cap, "gemm_skinny_kernel<%d>", t[1]);
         return SG_OK;
     }
-    snprintf(buf, cap, "gemm_mfma_kernel<%d, %d, %d, %s, %s, %s, %s>", t[0], t[1], t[2], t[3] ? "true" : "false", t[4] ? "true" : "false",
-             t[5] ? "true" : "false", t[6] ? "true" : "false");
+    snprintf(buf, cap, "gemm_mfma_kernel<%d, %d, %d, %s, %s, %s, %s, %s>", t[0], t[1], t[2], t[3] ? "true" : "false", t[4] ? "true" : "false",
+             t[5] ? "true" : "false", t[6] ? "true" : "false", t[7] ? "true" : "false");
     return SG_OK;
 }
 

@@ -682,7 +682,7 @@ def test_gemm_direct_write_out_with_special_bias_values(ctx, with_res):
     ctx.check(lib.sg_gemm(ctx.handle, 0, 0, C.byref(ac), C.byref(bc), C.byref(oc), C.byref(epi)))
     name = C.create_string_buffer(128)
     lib.sg_gemm_last_kernel_name(ctx.handle, name, 128)
-    assert b"false, false>" in name.value, f"expected an unguarded instantiation, got {name.value}"
+    assert b"false, false, true>" in name.value, f"expected an unguarded instantiation with the direct write-out, got {name.value}"
     got = out.numpy()
     with np.errstate(all="ignore"):
         want = a.astype(np.float64) @ b.astype(np.float64) + bias.astype(np.float64) + (res if with_res else 0.0)
@@ -951,14 +951,14 @@ def test_last_product_kernel_name(ctx):
     rng = np.random.default_rng(3)
     a, b = dev(ctx, rng.standard_normal((256, 64)).astype(np.float32)), dev(ctx, rng.standard_normal((64, 128)).astype(np.float32))
     a.matmul(b).eval(ctx)
-    assert last() == "gemm_mfma_kernel<64, 64, 2, true, true, false, false>", last()
+    assert last() == "gemm_mfma_kernel<64, 64, 2, true, true, false, false, true>", last()   # unguarded, plain product: the direct write-out
     dev(ctx, rng.standard_normal((70, 33)).astype(np.float32)).matmul(dev(ctx, rng.standard_normal((33, 19)).astype(np.float32))).eval(ctx)
-    assert last().endswith("true, false>") and ", true, true, true, false>" in last(), last()   # guarded loads
+    assert ", true, true, true, false, false>" in last(), last()   # guarded loads
     dev(ctx, rng.standard_normal((70, 33)).astype(np.float32)).matmul(dev(ctx, rng.standard_normal((33, 9)).astype(np.float32))).eval(ctx)
     assert last() == "gemm_skinny_kernel<16>", last()   # at most 16 output columns: a wavefront per output row
     dev(ctx, rng.standard_normal((70, 33)).astype(np.float32)).matmul(dev(ctx, rng.standard_normal((33, 2)).astype(np.float32))).eval(ctx)
     assert last() == "gemm_skinny_kernel<4>", last()
-    for c, want in ((64, "gemm_mfma_kernel<64, 64, 2, true, true, false, true>"), (5, "true, true, true, true>")):
+    for c, want in ((64, "gemm_mfma_kernel<64, 64, 2, true, true, false, true, true>"), (5, "true, true, true, true, false>")):
         x = S.Tensor.from_numpy(ctx, rng.standard_normal((4, 8, 8, c)).astype(np.float32))
         f = S.Tensor.from_numpy(ctx, rng.standard_normal((3, 3, c, 64)).astype(np.float32))
         out = S.Tensor.uninit(ctx, [4, 8, 8, 64])
